@@ -19,10 +19,22 @@ from .sequence import Sequence
 
 
 class BlockManager:
-    def __init__(self, num_blocks: int, block_size: int, watermark_blocks: int = 0) -> None:
+    def __init__(
+        self,
+        num_blocks: int,
+        block_size: int,
+        watermark_blocks: int = 0,
+        num_state_slots: int = 0,
+    ) -> None:
         self.num_blocks = num_blocks
         self.block_size = block_size
         self.watermark_blocks = watermark_blocks
+        # Recurrent-state slots (0 = the model keeps no per-sequence state):
+        # one slot per live sequence, handed out with its first blocks and
+        # reused LIFO like the blocks.  What a reused slot still holds is
+        # ignored: a sequence's first step starts its state from zero.
+        self.num_state_slots = num_state_slots
+        self._free_slots: List[int] = list(range(num_state_slots - 1, -1, -1))
         # LIFO free list: recently-freed blocks are re-used first (their cache
         # lines may still be resident in L2).
         self._free: List[int] = list(range(num_blocks - 1, -1, -1))
@@ -50,6 +62,8 @@ class BlockManager:
     def can_grow(self, seq: Sequence, target_len: int, respect_watermark: bool = False) -> bool:
         need = self.blocks_needed(seq, target_len)
         reserve = self.watermark_blocks if respect_watermark else 0
+        if self.num_state_slots and seq.state_slot < 0 and not self._free_slots:
+            return False
         return need <= len(self._free) - reserve
 
     # -- mutation ------------------------------------------------------------
@@ -60,9 +74,20 @@ class BlockManager:
             raise RuntimeError(
                 f"out of KV blocks: need {need}, free {len(self._free)}"
             )
+        if self.num_state_slots and seq.state_slot < 0:
+            if not self._free_slots:
+                raise RuntimeError("out of recurrent-state slots")
+            seq.state_slot = self._free_slots.pop()
         for _ in range(need):
             seq.block_table.append(self._free.pop())
+
+    @property
+    def num_free_state_slots(self) -> int:
+        return len(self._free_slots)
 
     def free(self, seq: Sequence) -> None:
         self._free.extend(reversed(seq.block_table))
         seq.block_table = []
+        if seq.state_slot >= 0:
+            self._free_slots.append(seq.state_slot)
+            seq.state_slot = -1

@@ -44,6 +44,9 @@ class EngineConfig:
     # Watermark of blocks kept free when admitting prefills.
     watermark_blocks: int = 8
     max_model_len: int = 4096
+    # Recurrent-state slots for models with recurrent layers (0 = one per
+    # max_num_seqs); ignored by models that keep only paged K/V.
+    num_state_slots: int = 0
     # Engine identity.
     engine_id: str = "engine-0"
     gpu_id: int = 0

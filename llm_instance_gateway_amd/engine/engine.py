@@ -56,6 +56,8 @@ class LLMEngine:
         # finished sequences ready for collection by the front door
         self._finished: List[Sequence] = []
         self._step_count = 0
+        # request_id -> Sequence of teacher-forced replays (replay_step)
+        self._replay_live: Dict[str, Sequence] = {}
         # adapter manager attaches itself here (lora.manager.AdapterManager)
         self.adapter_manager = None
         # callback(seq, token_id) fired on every generated token (streaming)
@@ -137,6 +139,38 @@ class LLMEngine:
         self._finished.extend(finished)
         self._step_count += 1
         return finished
+
+    # -- teacher-forced replay ----------------------------------------------------
+    def replay_step(self, entries, end=()) -> Dict[str, torch.Tensor]:
+        """Run one step over given tokens instead of sampled ones.
+
+        `entries`: [(request_id, next_token_ids, wanted_offsets)], all run as
+        ONE batch through the scheduler's block/slot bookkeeping and the
+        runner's step; a request is admitted at its first entry and may skip
+        steps.  `end`: request ids finished after this step (their blocks and
+        state slot go back to the pools).  Returns request_id -> fp32 logits
+        [len(wanted_offsets), vocab] for entries that asked for any."""
+        live = self._replay_live
+        plan = []
+        for rid, tokens, want in entries:
+            seq = live.get(rid)
+            if seq is None:
+                seq = Sequence([], sampling=SamplingParams(max_new_tokens=0), request_id=rid)
+                live[rid] = seq
+            seq.extend_prompt(list(tokens))
+            plan.append((seq, len(tokens), list(want)))
+        out = self.scheduler.schedule_forced(plan)
+        by_seq = self.runner.execute_replay(out)
+        res = {}
+        for seq, _, want in plan:
+            if want:
+                res[seq.request_id] = by_seq[seq.seq_id]
+        for rid in end:
+            seq = live.pop(rid, None)
+            if seq is not None:
+                self.scheduler.release(seq)
+        self._step_count += 1
+        return res
 
     def has_work(self) -> bool:
         return self.scheduler.has_work()

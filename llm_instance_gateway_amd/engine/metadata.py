@@ -65,6 +65,18 @@ class BatchMeta:
     # own so graph replay and a concurrent eager prefill never share u).
     lora_ws: Optional[torch.Tensor] = None
 
+    # Models with heterogeneous mixers (general-size attention, recurrent
+    # layers) address the flat batch per token and per sequence instead of
+    # per partition; built only when the model asks (needs_seq_tables).
+    # All sequences of the step, prefill portions first, then decodes:
+    seq_block_tables: Optional[torch.Tensor] = None  # [S, max_blocks] int32
+    tok_seq: Optional[torch.Tensor] = None    # [T] int32 row of the above; -1 = pad row
+    seg_start: Optional[torch.Tensor] = None  # [S] int32 first flat row of the sequence
+    seg_len: Optional[torch.Tensor] = None    # [S] int32 tokens it brings this step
+    seg_slot: Optional[torch.Tensor] = None   # [S] int32 recurrent-state slot
+    seg_fresh: Optional[torch.Tensor] = None  # [S] int32 1 = starts at position 0
+    max_seg_len: int = 0                      # host-side max of seg_len
+
     @property
     def num_tokens(self) -> int:
         return self.num_prefill_tokens + self.num_decode_tokens

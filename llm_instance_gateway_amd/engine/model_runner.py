@@ -27,30 +27,23 @@ log = logging.getLogger(__name__)
 
 
 def build_model(cfg: ModelConfig, device, dtype, tp=None):
-    if cfg.is_moe:
-        from ..models.mixtral import MixtralForCausalLM
+    """Instantiate the class registered for cfg.architecture (and load its
+    checkpoint when the config names a folder)."""
+    from ..models.registry import build_model as _build
 
-        return MixtralForCausalLM(cfg, device=device, dtype=dtype, tp=tp)
-    from ..models.llama import LlamaForCausalLM
-
-    return LlamaForCausalLM(cfg, device=device, dtype=dtype, tp=tp)
+    return _build(cfg, device, dtype, tp)
 
 
 def determine_num_kv_blocks(
-    config: EngineConfig, device: torch.device, tp_size: int = 1
+    config: EngineConfig, device: torch.device, tp_size: int = 1, elem_size: int = 2
 ) -> int:
     """Size the paged KV pool from free HBM after weights, honoring
     gpu_memory_utilization (the reference fleet runs vLLM at 0.95 —
     tools/dynamic-lora-sidecar/deployment.yaml:40)."""
     mc = config.model
-    bytes_per_block = (
-        mc.num_layers
-        * 2
-        * (mc.num_kv_heads // tp_size)
-        * config.block_size
-        * mc.head_dim
-        * 2  # bf16
-    )
+    # K+V of every layer that keeps a paged cache (recurrent layers keep a
+    # fixed-size state per slot instead, allocated separately)
+    bytes_per_block = max(1, mc.kv_elems_per_token(tp_size) * config.block_size * elem_size)
     if device.type == "cuda":
         free, total = torch.cuda.mem_get_info(device)
         budget = int(total * config.gpu_memory_utilization) - (total - free)
@@ -86,7 +79,9 @@ class ModelRunner:
             log.info("fp8 quantization: %d projection GEMMs converted", n_q)
         tp_size = tp.world_size if tp is not None else 1
         if self.device.type == "cuda":
-            n = determine_num_kv_blocks(config, self.device, tp_size)
+            n = determine_num_kv_blocks(
+                config, self.device, tp_size, torch.empty((), dtype=dtype).element_size()
+            )
             if n <= 0:
                 raise RuntimeError("no HBM left for KV cache after weights")
             config.num_kv_blocks = min(
@@ -94,19 +89,51 @@ class ModelRunner:
             )
         kvh = mc.num_kv_heads // tp_size
         # +1 scratch block: hipGraph decode padding rows write their K/V there
-        shape = (config.num_kv_blocks + 1, kvh, config.block_size, mc.head_dim)
-        self.kv_caches: List[Tuple[torch.Tensor, torch.Tensor]] = [
-            (
-                torch.zeros(shape, dtype=dtype, device=self.device),
-                torch.zeros(shape, dtype=dtype, device=self.device),
-            )
-            for _ in range(mc.num_layers)
-        ]
+        nblk = config.num_kv_blocks + 1
+        self.num_state_slots = 0
+        if hasattr(self.model, "cache_specs"):
+            # Heterogeneous stack: every layer declares what it keeps — paged
+            # K/V (key and value head sizes may differ) or an fp32 state
+            # vector per slot (+1 scratch slot for padding rows).
+            if mc.has_recurrent_state:
+                self.num_state_slots = config.num_state_slots or config.max_num_seqs
+            self.kv_caches = []
+            for spec in self.model.cache_specs():
+                if spec["kind"] == "kv":
+                    g = spec["kv_heads"]
+                    self.kv_caches.append(
+                        (
+                            torch.zeros((nblk, g, config.block_size, spec["k_dim"]), dtype=dtype, device=self.device),
+                            torch.zeros((nblk, g, config.block_size, spec["v_dim"]), dtype=dtype, device=self.device),
+                        )
+                    )
+                elif spec["kind"] == "state":
+                    self.kv_caches.append(
+                        (
+                            torch.zeros(
+                                (self.num_state_slots + 1, spec["width"]),
+                                dtype=torch.float32,
+                                device=self.device,
+                            ),
+                        )
+                    )
+                else:
+                    raise ValueError(f"unknown cache kind {spec['kind']!r}")
+        else:
+            shape = (nblk, kvh, config.block_size, mc.head_dim)
+            self.kv_caches: List[Tuple[torch.Tensor, torch.Tensor]] = [
+                (
+                    torch.zeros(shape, dtype=dtype, device=self.device),
+                    torch.zeros(shape, dtype=dtype, device=self.device),
+                )
+                for _ in range(mc.num_layers)
+            ]
         log.info(
-            "KV cache: %d blocks x %d tokens (%.1f GiB)",
+            "KV cache: %d blocks x %d tokens (%.1f GiB), %d state slots",
             config.num_kv_blocks,
             config.block_size,
-            2 * mc.num_layers * shape[0] * kvh * config.block_size * mc.head_dim * 2 / 2**30,
+            sum(t.numel() * t.element_size() for c in self.kv_caches for t in c) / 2**30,
+            self.num_state_slots,
         )
         self.adapter_manager = None
         self.graph_runner = None
@@ -122,6 +149,7 @@ class ModelRunner:
         self._use_graphs = (
             self.device.type == "cuda"
             and not config.enforce_eager
+            and getattr(self.model, "supports_decode_graphs", True)
             and (tp is None or _os.environ.get("LIG_TP_GRAPHS", "0") == "1")
         )
         # Mixed-step prefill/decode stream overlap — MEASURED DEAD END as a
@@ -314,9 +342,43 @@ class ModelRunner:
                     dev, non_blocking=True
                 )
 
+        ordered = prefills + decodes
+        # first flat row of every scheduled sequence (replay reads logits at
+        # offsets from it)
+        self._row_start = {}
+        r0 = 0
+        for ss in ordered:
+            self._row_start[ss.seq.seq_id] = r0
+            r0 += ss.num_tokens
+        if getattr(self.model, "needs_seq_tables", False):
+            # Per-token / per-sequence addressing for general-size attention
+            # and recurrent layers: one block-table row and one segment per
+            # scheduled sequence, prefill portions first, then decodes.
+            tok_seq: List[int] = []
+            s_start: List[int] = []
+            s_len: List[int] = []
+            s_slot: List[int] = []
+            s_fresh: List[int] = []
+            for si, ss in enumerate(ordered):
+                s_start.append(len(tok_seq))
+                s_len.append(ss.num_tokens)
+                s_slot.append(max(ss.seq.state_slot, 0))
+                s_fresh.append(1 if ss.seq.num_computed_tokens == 0 else 0)
+                tok_seq.extend([si] * ss.num_tokens)
+            tok_seq.extend([-1] * num_pad_tokens)
+
+            def i32(v: List[int]) -> torch.Tensor:
+                return torch.tensor(v, dtype=torch.int32).to(dev, non_blocking=True)
+
+            meta.seq_block_tables = pad_tables(p_bts + d_bts)
+            meta.tok_seq = i32(tok_seq)
+            meta.seg_start, meta.seg_len = i32(s_start), i32(s_len)
+            meta.seg_slot, meta.seg_fresh = i32(s_slot), i32(s_fresh)
+            meta.max_seg_len = max(s_len) if s_len else 0
+
         ids_t = torch.tensor(input_ids, dtype=torch.int64).to(dev, non_blocking=True)
         pos_t = torch.tensor(positions, dtype=torch.int64).to(dev, non_blocking=True)
-        return ids_t, pos_t, meta, sample_seqs, sample_idx, prefills + decodes
+        return ids_t, pos_t, meta, sample_seqs, sample_idx, ordered
 
     # -- one step --------------------------------------------------------------
     @torch.no_grad()
@@ -363,6 +425,38 @@ class ModelRunner:
         for ss in ordered:
             ss.seq.num_computed_tokens += ss.num_tokens
         return sampled
+
+    @torch.no_grad()
+    def execute_replay(self, out: SchedulerOutput) -> Dict[int, torch.Tensor]:
+        """Teacher-forced step: the same batch build and model forward as
+        `execute`, but nothing is sampled — returns, per sequence id, the
+        fp32 logits at the offsets its ScheduledSeq asks for, and advances
+        num_computed_tokens."""
+        if out.is_empty:
+            return {}
+        with gpu_range("build_batch"):
+            ids, pos, meta, _, _, ordered = self._build_batch(out)
+        with gpu_range("forward"), eager_tuned():
+            hidden = self.model(ids, pos, self.kv_caches, meta)
+        rows: List[int] = []
+        for ss in ordered:
+            base = self._row_start[ss.seq.seq_id]
+            for off in ss.logit_offsets or []:
+                if not 0 <= off < ss.num_tokens:
+                    raise ValueError("wanted logit offset outside the step's tokens")
+                rows.append(base + off)
+        res: Dict[int, torch.Tensor] = {}
+        if rows:
+            idx = torch.tensor(rows, dtype=torch.int64, device=self.device)
+            logits = self.model.compute_logits(hidden, idx)
+            at = 0
+            for ss in ordered:
+                n = len(ss.logit_offsets or [])
+                res[ss.seq.seq_id] = logits[at : at + n]
+                at += n
+        for ss in ordered:
+            ss.seq.num_computed_tokens += ss.num_tokens
+        return res
 
     def _execute_overlapped(self, out: SchedulerOutput) -> Optional[Dict[int, int]]:
         """Mixed-step stream overlap (ROADMAP r01 #9): the decode partition

@@ -34,6 +34,9 @@ from .sequence import Sequence, SequenceStatus
 class ScheduledSeq:
     seq: Sequence
     num_tokens: int  # 1 for decode; chunk size for prefill
+    # Teacher-forced replay: offsets within this step's tokens whose logits
+    # the caller wants (None = ordinary serving, sample at the end).
+    logit_offsets: Optional[List[int]] = None
 
     @property
     def is_prefill(self) -> bool:
@@ -57,8 +60,14 @@ class SchedulerOutput:
 class EngineScheduler:
     def __init__(self, config: EngineConfig, block_manager: Optional[BlockManager] = None) -> None:
         self.config = config
+        n_slots = 0
+        if config.model.has_recurrent_state:
+            n_slots = config.num_state_slots or config.max_num_seqs
         self.block_manager = block_manager or BlockManager(
-            config.num_kv_blocks, config.block_size, config.watermark_blocks
+            config.num_kv_blocks,
+            config.block_size,
+            config.watermark_blocks,
+            num_state_slots=n_slots,
         )
         self.waiting: Deque[Sequence] = deque()
         self.running: List[Sequence] = []
@@ -281,6 +290,48 @@ class EngineScheduler:
             token_budget -= chunk
 
         return out
+
+    # -- teacher-forced replay ---------------------------------------------------
+    def schedule_forced(
+        self, plan: List[Tuple[Sequence, int, Optional[List[int]]]]
+    ) -> SchedulerOutput:
+        """Build exactly the step the caller names: (sequence, number of its
+        next tokens, wanted logit offsets).  A sequence is admitted at its
+        first entry; blocks and a state slot come from the same pool as in
+        serving, and running out of either is an error here (a replay has no
+        one to preempt in favour of)."""
+        out = SchedulerOutput()
+        bm = self.block_manager
+        for seq, n, want in plan:
+            if n <= 0:
+                raise ValueError("a replayed entry brings at least one token")
+            if seq not in self.running:
+                if seq in self.waiting:
+                    self.waiting.remove(seq)
+                if len(self.running) >= self.config.max_num_seqs:
+                    raise RuntimeError("more live sequences than max_num_seqs")
+                seq.status = SequenceStatus.RUNNING
+                self.running.append(seq)
+            target = seq.num_computed_tokens + n
+            if target > seq.total_len:
+                raise ValueError("replayed entry runs past the sequence's known tokens")
+            if not bm.can_grow(seq, target):
+                raise RuntimeError(
+                    f"replay needs {bm.blocks_needed(seq, target)} KV blocks, "
+                    f"{bm.num_free_blocks} free (state slots free: {bm.num_free_state_slots})"
+                )
+            bm.grow(seq, target)
+            out.scheduled.append(ScheduledSeq(seq, n, list(want or [])))
+        return out
+
+    def release(self, seq: Sequence) -> None:
+        """Retire a sequence and give back its blocks and state slot."""
+        if seq in self.running:
+            self.running.remove(seq)
+        elif seq in self.waiting:
+            self.waiting.remove(seq)
+        seq.status = SequenceStatus.FINISHED
+        self.block_manager.free(seq)
 
     # -- post-step bookkeeping ---------------------------------------------------
     def finish_step(self, out: SchedulerOutput) -> List[Sequence]:

@@ -86,6 +86,10 @@ class Sequence:
         self.num_computed_tokens = 0
         # Paged KV block table (block ids owned by this sequence).
         self.block_table: List[int] = []
+        # Recurrent-state slot (models with recurrent layers; -1 = none yet).
+        # Owned by the block manager like the block table: handed out with
+        # the first blocks, given back by free().
+        self.state_slot: int = -1
         # Latency bookkeeping.
         self.arrival_time = arrival_time if arrival_time is not None else time.monotonic()
         self.first_scheduled_time: Optional[float] = None
@@ -125,6 +129,11 @@ class Sequence:
         return min(budget, self.total_len - self.num_computed_tokens)
 
     # -- transitions ---------------------------------------------------------
+    def extend_prompt(self, token_ids: List[int]) -> None:
+        """Teacher-forced replay: the request's next known tokens arrive
+        step by step instead of all at admission."""
+        self.prompt_token_ids.extend(token_ids)
+
     def append_token(self, token_id: int) -> None:
         self.output_token_ids.append(token_id)
         if self.first_token_time is None:
@@ -173,6 +182,7 @@ class Sequence:
         self.status = SequenceStatus.PREEMPTED
         self.num_computed_tokens = 0
         self.block_table = []
+        self.state_slot = -1  # recurrent state is recomputed from position 0
         self.num_preemptions += 1
 
     # -- SLO accounting -------------------------------------------------------

@@ -10,13 +10,28 @@ initialised randomly and the benchmark is synthetic-data.
 
 from __future__ import annotations
 
-from dataclasses import dataclass
-from typing import Optional
+from dataclasses import dataclass, field
+from typing import Any, Dict, List, Optional
+
+
+@dataclass
+class LayerSpec:
+    """One layer of a heterogeneous (hybrid) stack: which sequence mixer it
+    has ('attention' keeps paged K/V, 'mingru' keeps a recurrent state
+    vector), the mixer's sizes and constants, and its feed-forward (None for
+    a layer without one)."""
+
+    type: str
+    mixer: Dict[str, Any] = field(default_factory=dict)
+    mlp: Optional[Dict[str, Any]] = None
 
 
 @dataclass
 class ModelConfig:
     name: str
+    # Model family; selects the model class and config reader
+    # (models/registry.py).
+    architecture: str = "llama"
     vocab_size: int = 128256
     hidden_size: int = 4096
     num_layers: int = 32
@@ -36,6 +51,13 @@ class ModelConfig:
     # experts; models/mixtral.py MoEBlock docstring).
     expert_parallel: bool = False
     dtype: str = "bfloat16"
+    # Heterogeneous stacks: per-layer specs (None = num_layers identical
+    # Llama-style layers), and the number of equal parts the RMS norms split
+    # a row into (1 = ordinary RMS norm).
+    layer_specs: Optional[List[LayerSpec]] = None
+    norm_groups: int = 1
+    # Folder with config.json + model.safetensors ("" = random init).
+    weights_path: str = ""
 
     @property
     def is_moe(self) -> bool:
@@ -45,6 +67,27 @@ class ModelConfig:
     def kv_bytes_per_token_per_layer(self) -> int:
         # K + V, bf16.
         return 2 * self.num_kv_heads * self.head_dim * 2
+
+    def kv_elems_per_token(self, tp_size: int = 1) -> int:
+        """K+V elements one token occupies across all layers that keep a
+        paged cache (recurrent layers keep none)."""
+        if self.layer_specs is None:
+            return self.num_layers * 2 * (self.num_kv_heads // tp_size) * self.head_dim
+        return sum(
+            (s.mixer["kv_heads"] // tp_size) * (s.mixer["dim"] + s.mixer["vdim"])
+            for s in self.layer_specs
+            if s.type == "attention"
+        )
+
+    def state_elems_per_seq(self) -> int:
+        """fp32 recurrent-state elements one live sequence occupies."""
+        if self.layer_specs is None:
+            return 0
+        return sum(s.mixer["width"] for s in self.layer_specs if s.type == "mingru")
+
+    @property
+    def has_recurrent_state(self) -> bool:
+        return self.state_elems_per_seq() > 0
 
     def num_params(self) -> int:
         """Approximate parameter count (dense path)."""
@@ -139,6 +182,13 @@ PRESETS = {
 
 
 def get_model_config(name: str) -> ModelConfig:
+    """A preset by name, or a model folder (config.json picks the family)."""
+    import os
+
+    if name not in PRESETS and os.path.isfile(os.path.join(name, "config.json")):
+        from .registry import config_from_dir
+
+        return config_from_dir(name)
     if name not in PRESETS:
         raise KeyError(f"unknown model preset {name!r}; have {sorted(PRESETS)}")
     return PRESETS[name]

@@ -316,3 +316,176 @@ def linear(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
         _EXT.skinny_gemm(out, x.contiguous(), weight, _stream())
         return out
     return torch.nn.functional.linear(x, weight)
+
+
+# -- hybrid-model mechanisms ---------------------------------------------------
+# Grouped RMS norm over an fp32 residual, xIELU, the minGRU scan and paged
+# attention for any head sizes live in the light ctypes library (ops/hybrid.py,
+# plain C ABI, built by one hipcc call).  Storage dtype is bf16 or fp32; the
+# math is fp32 either way.
+
+def _use_hybrid(t: torch.Tensor) -> bool:
+    if not t.is_cuda:
+        return False
+    return os.environ.get("LIG_FORCE_TORCH_OPS") != "1"
+
+
+def _hl():
+    from . import hybrid
+
+    return hybrid.lib()
+
+
+def _is_f32(t: torch.Tensor) -> int:
+    if t.dtype == torch.float32:
+        return 1
+    if t.dtype == torch.bfloat16:
+        return 0
+    raise TypeError(f"hybrid kernels take bf16 or fp32 storage, got {t.dtype}")
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def embed_group_norm(tokens, table, w, eps: float, groups: int) -> torch.Tensor:
+    """residual[r] = group_norm(table[tokens[r]]) * w, fp32."""
+    H = table.shape[1]
+    assert H % groups == 0
+    if _use_hybrid(table):
+        R = tokens.shape[0]
+        res = torch.empty(R, H, dtype=torch.float32, device=table.device)
+        _hl().lig_embed_group_norm(
+            _ptr(res), _ptr(table), _ptr(tokens), _ptr(w), float(eps), R, H,
+            groups, _is_f32(table), _stream(),
+        )
+        return res
+    return torch_ref.embed_group_norm(tokens, table, w, eps, groups)
+
+
+def group_norm(residual, w, eps: float, groups: int) -> torch.Tensor:
+    """fp32 residual -> normalised activations in w's dtype."""
+    R, H = residual.shape
+    assert residual.dtype == torch.float32 and H % groups == 0
+    if _use_hybrid(residual):
+        out = torch.empty(R, H, dtype=w.dtype, device=residual.device)
+        _hl().lig_group_norm(
+            _ptr(out), _ptr(residual), _ptr(w), float(eps), R, H, groups,
+            _is_f32(w), _stream(),
+        )
+        return out
+    return torch_ref.group_norm(residual, w, eps, groups, w.dtype)
+
+
+def post_add_pre_norm(residual, y, w_post, w_pre, eps: float, groups: int):
+    """residual += group_norm(y) * w_post (in place); returns
+    group_norm(residual) * w_pre in y's dtype (None when w_pre is None)."""
+    R, H = residual.shape
+    assert residual.dtype == torch.float32 and y.shape == residual.shape
+    if _use_hybrid(residual):
+        assert y.is_contiguous() and residual.is_contiguous()
+        out = None if w_pre is None else torch.empty_like(y)
+        _hl().lig_post_add_pre_norm(
+            _ptr(out), _ptr(residual), _ptr(y), _ptr(w_post), _ptr(w_pre),
+            float(eps), R, H, groups, _is_f32(y), _stream(),
+        )
+        return out
+    return torch_ref.post_add_pre_norm(residual, y, w_post, w_pre, eps, groups)
+
+
+def xielu(x: torch.Tensor, a_pos: float, a_neg: float) -> torch.Tensor:
+    if _use_hybrid(x):
+        assert x.is_contiguous()
+        out = torch.empty_like(x)
+        _hl().lig_xielu(
+            _ptr(out), _ptr(x), float(a_pos), float(a_neg), x.numel(),
+            _is_f32(x), _stream(),
+        )
+        return out
+    return torch_ref.xielu(x, a_pos, a_neg)
+
+
+def sigmoid_gate_mul(x: torch.Tensor, g: torch.Tensor) -> torch.Tensor:
+    """x *= sigmoid(g) in place; g may be a column-block view (row stride)."""
+    if _use_hybrid(x):
+        assert x.is_contiguous() and g.stride(-1) == 1 and g.shape == x.shape
+        R, C = x.shape
+        _hl().lig_sigmoid_gate_mul(
+            _ptr(x), _ptr(g), g.stride(0), R, C, _is_f32(x), _stream()
+        )
+        return x
+    return torch_ref.sigmoid_gate_mul(x, g)
+
+
+def mingru_scan(zxg, state, seg_start, seg_len, seg_slot, seg_fresh, max_len: int):
+    """minGRU over the segments of a flat batch.  zxg [R, 3W] holds the gate
+    and candidate pre-activations and the output gate; state [slots, W] fp32
+    is read (unless the segment starts its sequence) and updated in place.
+    Rows outside every segment are left untouched (undefined)."""
+    R, W3 = zxg.shape
+    W = W3 // 3
+    assert state.dtype == torch.float32 and state.shape[1] == W
+    if _use_hybrid(zxg):
+        assert zxg.is_contiguous()
+        out = torch.empty(R, W, dtype=zxg.dtype, device=zxg.device)
+        es = zxg.element_size()
+        base = zxg.data_ptr()
+        _hl().lig_mingru_scan(
+            _ptr(out), base, base + W * es, base + 2 * W * es, W3, _ptr(state),
+            _ptr(seg_start), _ptr(seg_len), _ptr(seg_slot), _ptr(seg_fresh),
+            seg_start.shape[0], int(max_len), W, _is_f32(zxg), _stream(),
+        )
+        return out
+    return torch_ref.mingru_scan(zxg, state, seg_start, seg_len, seg_slot, seg_fresh, W)
+
+
+def kv_scatter(k, v, k_cache, v_cache, slot_mapping) -> None:
+    """Write K [R, G*D] / V [R, G*Dv] rows (column-block views sharing one
+    row stride) into caches whose K and V head sizes may differ."""
+    if _use_hybrid(k):
+        nb, G, bs, D = k_cache.shape
+        Dv = v_cache.shape[-1]
+        assert k.stride(0) == v.stride(0) and k.stride(1) == 1 and v.stride(1) == 1
+        assert k.shape[1] == G * D and v.shape[1] == G * Dv
+        assert k_cache.dtype == k.dtype and slot_mapping.dtype == torch.int64
+        _hl().lig_kv_scatter(
+            _ptr(k), _ptr(v), k.stride(0), _ptr(k_cache), _ptr(v_cache),
+            _ptr(slot_mapping), k.shape[0], G, D, Dv, bs, _is_f32(k), _stream(),
+        )
+        return
+    torch_ref.kv_scatter(k, v, k_cache, v_cache, slot_mapping)
+
+
+def paged_attention_general(
+    q, k_cache, v_cache, block_tables, tok_seq, positions, scale: float,
+    num_heads: int, gate=None, temp_coef: float = 0.0, temp_every: float = 1.0,
+) -> torch.Tensor:
+    """Causal paged attention for any key/value head sizes; token r of the
+    flat batch attends keys 0..positions[r] of sequence tok_seq[r].  Optional
+    query temperature 1 + coef*ln(floor((p+1)/every)+1) and sigmoid output
+    gate.  q/gate may be column-block views with a row stride."""
+    if _use_hybrid(q):
+        nb, G, bs, D = k_cache.shape
+        Dv = v_cache.shape[-1]
+        R = q.shape[0]
+        assert q.shape[1] == num_heads * D and q.stride(1) == 1
+        assert num_heads % G == 0 and Dv <= 512
+        assert block_tables.dtype == torch.int32 and tok_seq.dtype == torch.int32
+        assert positions.dtype == torch.int64 and block_tables.is_contiguous()
+        if gate is not None:
+            assert gate.shape == (R, num_heads * Dv) and gate.stride(1) == 1
+        out = torch.empty(R, num_heads * Dv, dtype=q.dtype, device=q.device)
+        ev = float(temp_every)
+        ev_int = int(ev) if ev == int(ev) and ev >= 1 else 0
+        _hl().lig_paged_attention_general(
+            _ptr(out), _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache),
+            _ptr(block_tables), block_tables.shape[1], _ptr(tok_seq),
+            _ptr(positions), _ptr(gate), 0 if gate is None else gate.stride(0),
+            float(scale), float(temp_coef), ev, ev_int, R, num_heads, G, D, Dv,
+            bs, _is_f32(q), _stream(),
+        )
+        return out
+    return torch_ref.paged_attention_general(
+        q, k_cache, v_cache, block_tables, tok_seq, positions, scale, num_heads,
+        gate, temp_coef, temp_every,
+    )

@@ -1,0 +1,193 @@
+// Paged causal attention for any head sizes, bf16 or fp32 storage, fp32
+// scores and softmax, gfx950.
+//
+// Serves the shapes the MFMA kernels do not: key size != value size, sizes
+// that are not 64/128, fp32 caches.  One wave per (token, query head) walks
+// the sequence's pages 64 keys at a time: lane j scores key j against the
+// query held in LDS, the wave keeps a running max / sum (online softmax),
+// then the lanes switch to value columns and accumulate sum_j p_j V[j, :].
+// Prompt portions and single decoded tokens go through the same walk: a
+// token at position p sees keys 0..p of its own sequence, whatever else is
+// in the flat batch.
+//
+// Optional per-position query temperature
+//   tau(p) = 1 + coef * ln(floor((p + 1) / every) + 1)
+// multiplies the score (same as scaling q), and an optional output gate
+// multiplies the result element-wise by sigmoid(gate) before it is stored.
+//
+// Cache layout: K [blocks, G, BS, D], V [blocks, G, BS, Dv].
+
+#include "elem_types.h"
+
+#define ATT_MAX_DV_PER_LANE 8  // Dv <= 512
+
+template <typename T>
+__global__ void paged_attention_general_kernel(
+    T* __restrict__ out,  // [R, H * Dv]
+    const T* __restrict__ q, long q_stride,
+    const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+    const int* __restrict__ block_tables, int max_blocks,
+    const int* __restrict__ tok_seq,        // [R], -1 = padding row
+    const int64_t* __restrict__ positions,  // [R]
+    const T* __restrict__ gate, long gate_stride, float scale, float temp_coef,
+    float temp_every, int temp_every_int, int H, int G, int D, int Dv, int BS) {
+  extern __shared__ __align__(16) float smem[];
+  float* q_s = smem;                       // [D], padded to an even count
+  float* p_s = smem + ((D + 1) & ~1);      // [64]
+  long* voff_s = reinterpret_cast<long*>(p_s + WAVE_SIZE);  // [64]
+
+  const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int seq = tok_seq[r];
+  T* orow = out + (size_t)r * H * Dv + (size_t)h * Dv;
+  if (seq < 0) {
+    for (int d = lane; d < Dv; d += WAVE_SIZE) st(orow + d, 0.f);
+    return;
+  }
+  const long pos = positions[r];
+  const int ctx = (int)pos + 1;
+  const int g = h / (H / G);
+  const int* bt = block_tables + (size_t)seq * max_blocks;
+
+  float tau = 1.f;
+  if (temp_coef != 0.f) {
+    const float n = temp_every_int > 0
+                        ? (float)((pos + 1) / temp_every_int)
+                        : floorf((float)(pos + 1) / temp_every);
+    tau = 1.f + temp_coef * logf(n + 1.f);
+  }
+  const float sc = scale * tau;
+
+  const T* qrow = q + (size_t)r * q_stride + (size_t)h * D;
+  for (int d = lane; d < D; d += WAVE_SIZE) q_s[d] = ld(qrow + d);
+  __syncthreads();
+
+  float m = -INFINITY, l = 0.f;
+  float acc[ATT_MAX_DV_PER_LANE];
+#pragma unroll
+  for (int i = 0; i < ATT_MAX_DV_PER_LANE; ++i) acc[i] = 0.f;
+
+  for (int j0 = 0; j0 < ctx; j0 += WAVE_SIZE) {
+    const int j = j0 + lane;
+    const bool valid = j < ctx;
+    float score = -INFINITY;
+    long voff = 0;
+    if (valid) {
+      const long blk = bt[j / BS];
+      const int off = j % BS;
+      const T* krow = k_cache + ((blk * G + g) * BS + off) * (long)D;
+      voff = ((blk * G + g) * BS + off) * (long)Dv;
+      float dot = 0.f;
+      for (int d = 0; d < D; ++d) dot += q_s[d] * ld(krow + d);
+      score = dot * sc;
+    }
+    const float m_new = fmaxf(m, wave_reduce_max(score));  // finite: key j0 is valid
+    const float p = valid ? expf(score - m_new) : 0.f;
+    const float alpha = expf(m - m_new);                   // 0 on the first tile
+    l = l * alpha + wave_reduce_sum(p);
+    m = m_new;
+    __syncthreads();  // previous tile's readers are done
+    p_s[lane] = p;
+    voff_s[lane] = voff;
+    __syncthreads();
+    const int nv = min(WAVE_SIZE, ctx - j0);
+#pragma unroll
+    for (int i = 0; i < ATT_MAX_DV_PER_LANE; ++i) {
+      const int d = lane + i * WAVE_SIZE;
+      if (d < Dv) {
+        float a = acc[i] * alpha;
+        for (int jj = 0; jj < nv; ++jj) a += p_s[jj] * ld(v_cache + voff_s[jj] + d);
+        acc[i] = a;
+      }
+    }
+  }
+  const float inv_l = 1.f / l;
+#pragma unroll
+  for (int i = 0; i < ATT_MAX_DV_PER_LANE; ++i) {
+    const int d = lane + i * WAVE_SIZE;
+    if (d < Dv) {
+      float o = acc[i] * inv_l;
+      if (gate != nullptr)
+        o *= sigmoid_f32(ld(gate + (size_t)r * gate_stride + (size_t)h * Dv + d));
+      st(orow + d, o);
+    }
+  }
+}
+
+// Scatter this step's K and V rows (column blocks of a fused projection
+// output, row stride `src_stride`) into the paged caches.
+template <typename T>
+__global__ void kv_scatter_kernel(const T* __restrict__ k, const T* __restrict__ v,
+                                  long src_stride, T* __restrict__ k_cache,
+                                  T* __restrict__ v_cache,
+                                  const int64_t* __restrict__ slot_mapping,
+                                  int R, int G, int D, int Dv, int BS) {
+  const int per_row = G * (D + Dv);
+  const long total = (long)R * per_row;
+  for (long idx = blockIdx.x * (long)blockDim.x + threadIdx.x; idx < total;
+       idx += gridDim.x * (long)blockDim.x) {
+    const long t = idx / per_row;
+    const int e = (int)(idx - t * per_row);
+    const int64_t slot = slot_mapping[t];
+    if (slot < 0) continue;
+    const long blk = slot / BS;
+    const int off = (int)(slot % BS);
+    if (e < G * D) {
+      const int g = e / D, d = e % D;
+      k_cache[((blk * G + g) * BS + off) * (long)D + d] = k[t * src_stride + e];
+    } else {
+      const int e2 = e - G * D;
+      const int g = e2 / Dv, d = e2 % Dv;
+      v_cache[((blk * G + g) * BS + off) * (long)Dv + d] = v[t * src_stride + e2];
+    }
+  }
+}
+
+extern "C" {
+
+void lig_paged_attention_general(
+    void* out, const void* q, long q_stride, const void* k_cache,
+    const void* v_cache, const int* block_tables, int max_blocks,
+    const int* tok_seq, const int64_t* positions, const void* gate,
+    long gate_stride, float scale, float temp_coef, float temp_every,
+    int temp_every_int, int R, int H, int G, int D, int Dv, int BS, int is_f32,
+    hipStream_t s) {
+  if (R <= 0) return;
+  dim3 grid(R, H), block(WAVE_SIZE);
+  const size_t smem = (size_t)(((D + 1) & ~1) + WAVE_SIZE) * sizeof(float) + WAVE_SIZE * sizeof(long);
+  if (is_f32)
+    hipLaunchKernelGGL(paged_attention_general_kernel<float>, grid, block, smem,
+                       s, (float*)out, (const float*)q, q_stride,
+                       (const float*)k_cache, (const float*)v_cache,
+                       block_tables, max_blocks, tok_seq, positions,
+                       (const float*)gate, gate_stride, scale, temp_coef,
+                       temp_every, temp_every_int, H, G, D, Dv, BS);
+  else
+    hipLaunchKernelGGL(paged_attention_general_kernel<bf16s>, grid, block, smem,
+                       s, (bf16s*)out, (const bf16s*)q, q_stride,
+                       (const bf16s*)k_cache, (const bf16s*)v_cache,
+                       block_tables, max_blocks, tok_seq, positions,
+                       (const bf16s*)gate, gate_stride, scale, temp_coef,
+                       temp_every, temp_every_int, H, G, D, Dv, BS);
+}
+
+void lig_kv_scatter(const void* k, const void* v, long src_stride,
+                    void* k_cache, void* v_cache, const int64_t* slot_mapping,
+                    int R, int G, int D, int Dv, int BS, int is_f32,
+                    hipStream_t s) {
+  const long total = (long)R * G * (D + Dv);
+  if (total <= 0) return;
+  long gl = (total + 255) / 256;
+  const int grid = (int)(gl > 65535 ? 65535 : gl);
+  if (is_f32)
+    hipLaunchKernelGGL(kv_scatter_kernel<float>, dim3(grid), dim3(256), 0, s,
+                       (const float*)k, (const float*)v, src_stride,
+                       (float*)k_cache, (float*)v_cache, slot_mapping, R, G, D,
+                       Dv, BS);
+  else
+    hipLaunchKernelGGL(kv_scatter_kernel<bf16s>, dim3(grid), dim3(256), 0, s,
+                       (const bf16s*)k, (const bf16s*)v, src_stride,
+                       (bf16s*)k_cache, (bf16s*)v_cache, slot_mapping, R, G, D,
+                       Dv, BS);
+}
+
+}  // extern "C"

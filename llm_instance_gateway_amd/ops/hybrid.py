@@ -1,0 +1,107 @@
+"""Light native library for the hybrid-model kernels (grouped RMS norm, xIELU,
+minGRU scan, general-size paged attention).
+
+These kernels expose a plain C ABI and need no torch headers, so they are
+compiled by one direct ``hipcc -shared`` call (seconds, not the minutes the
+torch extension takes) into ``llm_instance_gateway_amd/_hybrid.so`` and
+loaded with ctypes.  A model that needs only these kernels can therefore be
+served from a fresh checkout after a short first-use build; nothing else is
+compiled for it.
+
+``build()`` always compiles; ``lib()`` loads what is built and builds only
+when nothing is there (guarded by a file lock so concurrent processes build
+once).
+"""
+
+from __future__ import annotations
+
+import ctypes
+import fcntl
+import os
+import shutil
+import subprocess
+import tempfile
+from pathlib import Path
+from typing import Optional
+
+PKG = Path(__file__).resolve().parent.parent
+CSRC = Path(__file__).resolve().parent / "csrc"
+# Sources of the light library; setup.py leaves these out of the torch
+# extension.
+SOURCES = ["group_norm.hip", "xielu.hip", "mingru.hip", "attention_general.hip"]
+SO_PATH = PKG / "_hybrid.so"
+
+_LIB: Optional[ctypes.CDLL] = None
+
+
+def _hipcc() -> str:
+    for cand in (shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.exists(cand):
+            return cand
+    raise RuntimeError("hipcc not found; cannot build the hybrid kernel library")
+
+
+def build() -> Path:
+    """Compile the light library for gfx950 (atomic replace of the .so)."""
+    fd, tmp = tempfile.mkstemp(prefix="._hybrid-", suffix=".so", dir=str(PKG))
+    os.close(fd)
+    cmd = [
+        _hipcc(), "-O3", "-std=c++17", "--offload-arch=gfx950",
+        "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+        "-shared", "-fPIC", "-o", tmp,
+    ] + [str(CSRC / s) for s in SOURCES]
+    try:
+        subprocess.run(cmd, check=True, cwd=str(CSRC), stdout=subprocess.PIPE,
+                       stderr=subprocess.PIPE)
+        os.chmod(tmp, 0o755)
+        os.replace(tmp, SO_PATH)
+    except subprocess.CalledProcessError as e:
+        raise RuntimeError(
+            "building the hybrid kernel library failed:\n" + e.stderr.decode(errors="replace")[-4000:]
+        ) from None
+    finally:
+        if os.path.exists(tmp):
+            os.unlink(tmp)
+    return SO_PATH
+
+
+def _declare(lib: ctypes.CDLL) -> None:
+    p, i, l, f = ctypes.c_void_p, ctypes.c_int, ctypes.c_long, ctypes.c_float
+    sigs = {
+        "lig_embed_group_norm": [p, p, p, p, f, i, i, i, i, p],
+        "lig_group_norm": [p, p, p, f, i, i, i, i, p],
+        "lig_post_add_pre_norm": [p, p, p, p, p, f, i, i, i, i, p],
+        "lig_xielu": [p, p, f, f, l, i, p],
+        "lig_sigmoid_gate_mul": [p, p, l, i, i, i, p],
+        "lig_mingru_scan": [p, p, p, p, l, p, p, p, p, p, i, i, i, i, p],
+        "lig_paged_attention_general": [
+            p, p, l, p, p, p, i, p, p, p, l, f, f, f, i, i, i, i, i, i, i, i, p,
+        ],
+        "lig_kv_scatter": [p, p, l, p, p, p, i, i, i, i, i, i, p],
+    }
+    for name, args in sigs.items():
+        fn = getattr(lib, name)
+        fn.argtypes = args
+        fn.restype = None
+
+
+def lib() -> ctypes.CDLL:
+    global _LIB
+    if _LIB is not None:
+        return _LIB
+    if not SO_PATH.exists():
+        lock = PKG / "._hybrid.lock"
+        with open(lock, "w") as lf:
+            fcntl.flock(lf, fcntl.LOCK_EX)
+            try:
+                if not SO_PATH.exists():
+                    build()
+            finally:
+                fcntl.flock(lf, fcntl.LOCK_UN)
+    _LIB = ctypes.CDLL(str(SO_PATH))
+    _declare(_LIB)
+    return _LIB
+
+
+def available() -> bool:
+    return SO_PATH.exists()

@@ -211,3 +211,123 @@ def sgmv_expand(
         s = int(slots[t])
         if s >= 0:
             y[t] += (b_stack[s].float() @ u[t].float() * scaling).to(y.dtype)
+
+
+# -- hybrid-model mechanisms (grouped norm, xIELU, minGRU, general attention) --
+# Same rounding points as the HIP kernels: fp32 math, results cast to the
+# activation dtype; the residual stream and the recurrent state stay fp32.
+
+def _group_scale(x: torch.Tensor, groups: int, eps: float) -> torch.Tensor:
+    R, H = x.shape
+    xg = x.float().view(R, groups, H // groups)
+    return (xg / torch.sqrt(xg.pow(2).mean(dim=-1, keepdim=True) + eps)).view(R, H)
+
+
+def embed_group_norm(tokens, table, w, eps: float, groups: int) -> torch.Tensor:
+    return _group_scale(table[tokens], groups, eps) * w.float()
+
+
+def group_norm(residual, w, eps: float, groups: int, out_dtype) -> torch.Tensor:
+    return (_group_scale(residual, groups, eps) * w.float()).to(out_dtype)
+
+
+def post_add_pre_norm(residual, y, w_post, w_pre, eps: float, groups: int):
+    residual.add_(_group_scale(y, groups, eps) * w_post.float())
+    if w_pre is None:
+        return None
+    return (_group_scale(residual, groups, eps) * w_pre.float()).to(y.dtype)
+
+
+def xielu(x: torch.Tensor, a_pos: float, a_neg: float) -> torch.Tensor:
+    z = x.float()
+    neg = a_neg * (torch.expm1(torch.clamp(z, max=0.0)) - z) + 0.5 * z
+    pos = a_pos * z * z + 0.5 * z
+    return torch.where(z > 0, pos, neg).to(x.dtype)
+
+
+def sigmoid_gate_mul(x: torch.Tensor, g: torch.Tensor) -> torch.Tensor:
+    return x.copy_((x.float() * torch.sigmoid(g.float())).to(x.dtype))
+
+
+def mingru_scan(zxg, state, seg_start, seg_len, seg_slot, seg_fresh, W: int):
+    """zxg [R, 3W] = (gate pre-activation | candidate pre-activation | output
+    gate); state [slots, W] fp32, updated in place."""
+    R = zxg.shape[0]
+    out = torch.zeros(R, W, dtype=zxg.dtype, device=zxg.device)
+    z = torch.sigmoid(zxg[:, :W].float())
+    u = zxg[:, W : 2 * W].float()
+    cand = torch.where(u >= 0, u + 0.5, torch.sigmoid(u))
+    g = zxg[:, 2 * W :].float()
+    og = g * torch.sigmoid(g)
+    for s0, n, slot, fresh in zip(
+        seg_start.tolist(), seg_len.tolist(), seg_slot.tolist(), seg_fresh.tolist()
+    ):
+        if n <= 0:
+            continue
+        S = torch.zeros(W, dtype=torch.float32, device=zxg.device) if fresh else state[slot].clone()
+        for t in range(s0, s0 + n):
+            S = (1.0 - z[t]) * S + z[t] * cand[t]
+            out[t] = (S * og[t]).to(out.dtype)
+        state[slot] = S
+    return out
+
+
+def kv_scatter(k, v, k_cache, v_cache, slot_mapping) -> None:
+    nb, G, bs, D = k_cache.shape
+    Dv = v_cache.shape[-1]
+    T = k.shape[0]
+    ok = slot_mapping >= 0
+    blk = torch.div(slot_mapping, bs, rounding_mode="floor")[ok]
+    off = (slot_mapping % bs)[ok]
+    k_cache[blk, :, off, :] = k.reshape(T, G, D)[ok].to(k_cache.dtype)
+    v_cache[blk, :, off, :] = v.reshape(T, G, Dv)[ok].to(v_cache.dtype)
+
+
+def query_temperature(positions: torch.Tensor, coef: float, every: float) -> torch.Tensor:
+    n = torch.floor((positions.double() + 1.0) / every)
+    return (1.0 + coef * torch.log(n + 1.0)).float()
+
+
+def paged_attention_general(
+    q, k_cache, v_cache, block_tables, tok_seq, positions, scale: float,
+    num_heads: int, gate=None, temp_coef: float = 0.0, temp_every: float = 1.0,
+):
+    """q [R, H*D] (may be a strided view); token r belongs to sequence row
+    tok_seq[r] of block_tables (-1: padding row) and sees keys 0..positions[r]."""
+    R = q.shape[0]
+    nb, G, bs, D = k_cache.shape
+    Dv = v_cache.shape[-1]
+    H = num_heads
+    out = torch.zeros(R, H * Dv, dtype=q.dtype, device=q.device)
+    seqs = tok_seq.tolist()
+    pos = positions.tolist()
+    tau = (
+        query_temperature(positions, temp_coef, temp_every)
+        if temp_coef != 0.0
+        else torch.ones(R, dtype=torch.float32, device=q.device)
+    )
+    r = 0
+    while r < R:
+        s = seqs[r]
+        e = r + 1
+        while e < R and seqs[e] == s:
+            e += 1
+        if s >= 0:
+            L = max(pos[r:e]) + 1
+            nblk = (L + bs - 1) // bs
+            ids = block_tables[s, :nblk].long()
+            k = k_cache[ids].permute(0, 2, 1, 3).reshape(nblk * bs, G, D)[:L].float()
+            v = v_cache[ids].permute(0, 2, 1, 3).reshape(nblk * bs, G, Dv)[:L].float()
+            kf = k.repeat_interleave(H // G, dim=1).permute(1, 0, 2)  # [H, L, D]
+            vf = v.repeat_interleave(H // G, dim=1).permute(1, 0, 2)
+            qf = q[r:e].float().reshape(e - r, H, D).permute(1, 0, 2)  # [H, n, D]
+            sc = torch.bmm(qf, kf.transpose(1, 2)) * (scale * tau[r:e])[None, :, None]
+            keyp = torch.arange(L, device=q.device)[None, :]
+            mask = keyp > positions[r:e, None]
+            sc.masked_fill_(mask[None], float("-inf"))
+            o = torch.bmm(torch.softmax(sc, dim=-1), vf).permute(1, 0, 2).reshape(e - r, H * Dv)
+            if gate is not None:
+                o = o * torch.sigmoid(gate[r:e].float())
+            out[r:e] = o.to(out.dtype)
+        r = e
+    return out

@@ -21,11 +21,19 @@ ROOT = Path(__file__).parent
 CSRC = ROOT / "llm_instance_gateway_amd" / "ops" / "csrc"
 RCSRC = ROOT / "llm_instance_gateway_amd" / "router" / "csrc"
 
+# Kernels with a plain C ABI that are built on their own by one hipcc call
+# (llm_instance_gateway_amd/ops/hybrid.py::SOURCES) stay out of the torch
+# extension.
+_light = (ROOT / "llm_instance_gateway_amd" / "ops" / "hybrid.py").read_text()
+LIGHT_SOURCES = set(
+    __import__("re").findall(r'"([a-z_]+\.hip)"', _light.split("SOURCES = [", 1)[1].split("]", 1)[0])
+)
+
 sources = sorted(
     str(p)
     for p in CSRC.glob("*.hip")
     # hipify writes shadow copies named *_hip.hip next to the originals
-    if not p.name.endswith("_hip.hip")
+    if not p.name.endswith("_hip.hip") and p.name not in LIGHT_SOURCES
 )
 
 # LIG_DEBUG=1: host-side index/range validation in the bindings (make
@@ -42,6 +50,9 @@ ext = CUDAExtension(
             "-O3",
             "-std=c++17",
             "--offload-arch=gfx950",
+            # no packed-fp32 VALU forms (hipcc's host pass warns that it does
+            # not know the feature; harmless)
+            "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
         ] + debug_flags,
     },
 )
