@@ -83,6 +83,23 @@ class DecodeGraphRunner:
         self.n_ut0 = self.h_ut0.numpy()
         self.n_ulen = self.h_ulen.numpy()
         self.n_uslot = self.h_uslot.numpy()
+        # Models that address the batch per sequence (general-size attention,
+        # recurrent layers): a decode step is B one-token segments, row i ==
+        # sequence i; only the state slot and the starts-here flag vary.
+        self.seq_tables = bool(getattr(runner.model, "needs_seq_tables", False))
+        if self.seq_tables:
+            ar = torch.arange(B, dtype=torch.int32, device=dev)
+            self.tok_seq = ar.clone()
+            self.seg_start = ar.clone()
+            self.seg_len = torch.ones(B, dtype=torch.int32, device=dev)
+            # scratch state slot for padding rows = one past the pool
+            self.scratch_slot = getattr(runner, "num_state_slots", 0)
+            self.seg_slot = torch.full((B,), self.scratch_slot, dtype=torch.int32, device=dev)
+            self.seg_fresh = torch.ones(B, dtype=torch.int32, device=dev)
+            self.h_sslot = torch.zeros(B, dtype=torch.int32, pin_memory=True)
+            self.h_sfresh = torch.ones(B, dtype=torch.int32, pin_memory=True)
+            self.n_sslot = self.h_sslot.numpy()
+            self.n_sfresh = self.h_sfresh.numpy()
         # scratch KV block for padding rows = last block of the (extended) pool
         self.scratch_block = runner.config.num_kv_blocks  # extra block id
         self.graphs: Dict[int, torch.cuda.CUDAGraph] = {}
@@ -97,13 +114,34 @@ class DecodeGraphRunner:
         profiles/r01_flash_decode_split.txt)."""
         from .. import ops
 
-        attn = self.runner.model.layers[0].self_attn
-        return ops.decode_nsplits(
-            B, attn.num_kv_heads, self.max_blocks * self.block_size
-        )
+        shape = self._attn_shape()
+        if shape is None:
+            return 1
+        return ops.decode_nsplits(B, shape[1], self.max_blocks * self.block_size)
+
+    def _attn_shape(self):
+        """(q heads, kv heads, head size) of the layers that run the split
+        paged-decode kernel; None when no layer does."""
+        model = self.runner.model
+        if hasattr(model, "decode_attention_shape"):
+            return model.decode_attention_shape()
+        attn = model.layers[0].self_attn
+        return attn.num_heads, attn.num_kv_heads, attn.head_dim
 
     def _meta(self, B: int) -> BatchMeta:
+        extra = {}
+        if self.seq_tables:
+            extra = dict(
+                seq_block_tables=self.block_tables[:B],
+                tok_seq=self.tok_seq[:B],
+                seg_start=self.seg_start[:B],
+                seg_len=self.seg_len[:B],
+                seg_slot=self.seg_slot[:B],
+                seg_fresh=self.seg_fresh[:B],
+                max_seg_len=1,
+            )
         return BatchMeta(
+            **extra,
             num_prefill_tokens=0,
             num_decode_tokens=B,
             slot_mapping=self.slot_mapping[:B],
@@ -122,7 +160,7 @@ class DecodeGraphRunner:
         model = self.runner.model
         hidden = model(self.ids[:B], self.pos[:B], self.runner.kv_caches, self._meta(B))
         idx = torch.arange(B, device=self.device)
-        return model.compute_logits(hidden, idx).to(torch.bfloat16)
+        return model.compute_logits(hidden, idx).to(self.runner.dtype)
 
     def capture(self, with_lora: bool) -> None:
         self.with_lora = with_lora
@@ -137,8 +175,8 @@ class DecodeGraphRunner:
         # earlier graphs pointing at freed memory).
         from .. import ops
 
-        attn = self.runner.model.layers[0].self_attn
-        hq, d = attn.num_heads, attn.head_dim
+        shape = self._attn_shape()
+        hq, d = (shape[0], shape[2]) if shape is not None else (0, 0)
         max_scratch = max(
             (B * hq * self._graph_nsplits(B) * (d + 2) for B in self.sizes),
             default=0,
@@ -208,6 +246,14 @@ class DecodeGraphRunner:
             n_ctx[i] = p + 1
             if self.with_lora:
                 n_lora[i] = slot_of(seq.lora_name) if seq.lora_name else -1
+            if self.seq_tables:
+                self.n_sslot[i] = max(seq.state_slot, 0)
+                self.n_sfresh[i] = 1 if p == 0 else 0
+        if self.seq_tables:
+            self.n_sslot[n:B] = self.scratch_slot
+            self.n_sfresh[n:B] = 1
+            self.seg_slot[:B].copy_(self.h_sslot[:B], non_blocking=True)
+            self.seg_fresh[:B].copy_(self.h_sfresh[:B], non_blocking=True)
         # padding rows
         if B > n:
             n_ids[n:B] = 0

@@ -266,6 +266,12 @@ class ModelRunner:
         # every transformer block reuse it; see profiles/r01_bench_kernel_stats.md).
         if prefills:
             use_mfma = self.device.type == "cuda" and self.config.model.head_dim in (64, 128)
+            if getattr(self.model, "needs_seq_tables", False):
+                # per-layer head sizes: the model says whether any layer runs
+                # the tiled kernel; none needs the per-token expansion
+                use_mfma = self.device.type == "cuda" and getattr(
+                    self.model, "needs_prefill_tiles", False
+                )
             if use_mfma:
                 # 64-row query tiles for the MFMA flash-prefill kernel.
                 ts: List[int] = []
@@ -280,7 +286,7 @@ class ModelRunner:
                 meta.prefill_tile_qstart = torch.tensor(tq, dtype=torch.int32).to(
                     dev, non_blocking=True
                 )
-            else:
+            elif not getattr(self.model, "needs_seq_tables", False):
                 ctx_tok: List[int] = []
                 n_per: List[int] = []
                 for ss in prefills:

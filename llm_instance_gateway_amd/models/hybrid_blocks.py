@@ -89,12 +89,40 @@ class GatedAttention(nn.Module):
         q, k, v = proj[:, :a], proj[:, a:b], proj[:, b:c]
         gate = proj[:, c:] if self.out_gate else None
         ops.kv_scatter(k, v, k_cache, v_cache, meta.slot_mapping)
-        o = ops.paged_attention_general(
-            q, k_cache, v_cache, meta.seq_block_tables, meta.tok_seq, positions,
-            self.scale, self.heads, gate=gate, temp_coef=self.temp_coef,
-            temp_every=self.temp_every,
-        )
+        if ops.mfma_attention_supported(proj.dtype, self.dim, self.vdim, proj.is_cuda):
+            o = self._attend_mfma(q, gate, positions, k_cache, v_cache, meta)
+        else:
+            o = ops.paged_attention_general(
+                q, k_cache, v_cache, meta.seq_block_tables, meta.tok_seq, positions,
+                self.scale, self.heads, gate=gate, temp_coef=self.temp_coef,
+                temp_every=self.temp_every,
+            )
         return F.linear(o, self.w_o)
+
+    def _attend_mfma(self, q, gate, positions, k_cache, v_cache, meta):
+        """bf16, key size == value size in {64, 128}: the MFMA flash-prefill
+        and paged-decode kernels do the softmax(QK^T)V; the temperature is
+        folded into q beforehand and the gate applied afterwards."""
+        qh = ops.temperature_scale_rows(q, positions, self.temp_coef, self.temp_every)
+        qh = qh.view(-1, self.heads, self.dim)
+        np_, nd = meta.num_prefill_tokens, meta.num_decode_tokens
+        out = torch.zeros_like(qh) if np_ + nd < qh.shape[0] else torch.empty_like(qh)
+        if np_ > 0:
+            out[:np_] = ops.paged_attention_prefill(
+                qh[:np_], k_cache, v_cache, meta.prefill_block_tables,
+                meta.prefill_query_start_locs, meta.prefill_context_lens, self.scale,
+                tile_seq=meta.prefill_tile_seq, tile_qstart=meta.prefill_tile_qstart,
+            )
+        if nd > 0:
+            out[np_ : np_ + nd] = ops.paged_attention_decode(
+                qh[np_ : np_ + nd], k_cache, v_cache, meta.decode_block_tables,
+                meta.decode_context_lens, self.scale, max_ctx=meta.max_decode_ctx,
+                nsplits=meta.decode_nsplits,
+            )
+        o = out.view(-1, self.heads * self.vdim)
+        if gate is not None:
+            ops.sigmoid_gate_mul(o, gate)
+        return o
 
 
 class MinGRU(nn.Module):

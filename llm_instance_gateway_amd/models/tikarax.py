@@ -95,9 +95,8 @@ class HybridLayer(nn.Module):
 class TikaraxForCausalLM(nn.Module):
     # the runner builds per-token sequence tables and per-sequence segments
     needs_seq_tables = True
-    # decode-only steps run eager (the hipGraph runner's static buffers do
-    # not carry segment tables yet)
-    supports_decode_graphs = False
+    # decode-only steps replay hipGraphs (one-token segments, static tables)
+    supports_decode_graphs = True
 
     def __init__(self, cfg: ModelConfig, device="cpu", dtype=torch.bfloat16, tp=None) -> None:
         super().__init__()
@@ -119,9 +118,32 @@ class TikaraxForCausalLM(nn.Module):
         self.layers = nn.ModuleList(
             [HybridLayer(s, H, device, dtype) for s in cfg.layer_specs]
         )
+        # any attention layer with bf16 and key size == value size in {64,128}
+        # runs the tiled MFMA prefill kernel and needs its 64-row query tiles
+        self.needs_prefill_tiles = any(
+            s.type == "attention"
+            and ops.mfma_attention_supported(
+                dtype, s.mixer["dim"], s.mixer["vdim"], self.device_.type == "cuda"
+            )
+            for s in cfg.layer_specs
+        )
         # test/debug hook: when a list, forward() appends the fp32 residual
         # stream after every layer
         self.capture_residuals: Optional[list] = None
+
+    def decode_attention_shape(self):
+        """(q heads, kv heads, head size) for sizing the split-decode scratch:
+        the largest among layers on the MFMA path, None if there is none."""
+        best = None
+        for layer in self.layers:
+            m = layer.mixer
+            if isinstance(m, GatedAttention) and ops.mfma_attention_supported(
+                self.dtype_, m.dim, m.vdim, self.device_.type == "cuda"
+            ):
+                cand = (m.heads, m.kv_heads, m.dim)
+                if best is None or cand[0] * cand[2] > best[0] * best[2]:
+                    best = cand
+        return best
 
     def cache_specs(self) -> List[dict]:
         return [layer.mixer.cache_spec() for layer in self.layers]

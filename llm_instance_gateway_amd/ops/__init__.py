@@ -489,3 +489,34 @@ def paged_attention_general(
         q, k_cache, v_cache, block_tables, tok_seq, positions, scale, num_heads,
         gate, temp_coef, temp_every,
     )
+
+
+def temperature_scale_rows(q, positions, coef: float, every: float) -> torch.Tensor:
+    """Contiguous copy of q [R, C] (may be a strided column block) with row r
+    multiplied by 1 + coef*ln(floor((positions[r]+1)/every)+1)."""
+    if _use_hybrid(q):
+        R, C = q.shape
+        assert q.stride(1) == 1 and positions.dtype == torch.int64
+        out = torch.empty(R, C, dtype=q.dtype, device=q.device)
+        ev = float(every)
+        ev_int = int(ev) if ev == int(ev) and ev >= 1 else 0
+        _hl().lig_temperature_scale_rows(
+            _ptr(out), _ptr(q), q.stride(0), _ptr(positions), float(coef), ev,
+            ev_int, R, C, _is_f32(q), _stream(),
+        )
+        return out
+    return torch_ref.temperature_scale_rows(q, positions, coef, every)
+
+
+def mfma_attention_supported(q_dtype, k_dim: int, v_dim: int, is_cuda: bool) -> bool:
+    """The MFMA flash-prefill / paged-decode kernels of the torch extension
+    serve bf16 caches with equal key and value head size 64 or 128."""
+    return (
+        is_cuda
+        and q_dtype == torch.bfloat16
+        and k_dim == v_dim
+        and k_dim in (64, 128)
+        and os.environ.get("LIG_FORCE_TORCH_OPS") != "1"
+        and os.environ.get("LIG_GENERAL_ATTENTION") != "1"
+        and native_available()
+    )

@@ -142,7 +142,50 @@ __global__ void kv_scatter_kernel(const T* __restrict__ k, const T* __restrict__
   }
 }
 
+// q_out[r, :] = q[r, :] * tau(position r): the query temperature applied
+// ahead of an attention kernel that takes one scalar scale.  Also packs the
+// strided q view (a column block of the fused projection) contiguously.
+template <typename T>
+__global__ void temperature_scale_rows_kernel(T* __restrict__ out,  // [R, C]
+                                              const T* __restrict__ q, long q_stride,
+                                              const int64_t* __restrict__ positions,
+                                              float temp_coef, float temp_every,
+                                              int temp_every_int, int C, long n) {
+  for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < n;
+       i += gridDim.x * (long)blockDim.x) {
+    const long r = i / C;
+    const int c = (int)(i - r * C);
+    float tau = 1.f;
+    if (temp_coef != 0.f) {
+      const long pos = positions[r];
+      const float m = temp_every_int > 0
+                          ? (float)((pos + 1) / temp_every_int)
+                          : floorf((float)(pos + 1) / temp_every);
+      tau = 1.f + temp_coef * logf(m + 1.f);
+    }
+    st(out + i, ld(q + r * q_stride + c) * tau);
+  }
+}
+
 extern "C" {
+
+void lig_temperature_scale_rows(void* out, const void* q, long q_stride,
+                                const int64_t* positions, float temp_coef,
+                                float temp_every, int temp_every_int, int R,
+                                int C, int is_f32, hipStream_t s) {
+  const long n = (long)R * C;
+  if (n <= 0) return;
+  long gl = (n + 255) / 256;
+  const int grid = (int)(gl > 65535 ? 65535 : gl);
+  if (is_f32)
+    hipLaunchKernelGGL(temperature_scale_rows_kernel<float>, dim3(grid),
+                       dim3(256), 0, s, (float*)out, (const float*)q, q_stride,
+                       positions, temp_coef, temp_every, temp_every_int, C, n);
+  else
+    hipLaunchKernelGGL(temperature_scale_rows_kernel<bf16s>, dim3(grid),
+                       dim3(256), 0, s, (bf16s*)out, (const bf16s*)q, q_stride,
+                       positions, temp_coef, temp_every, temp_every_int, C, n);
+}
 
 void lig_paged_attention_general(
     void* out, const void* q, long q_stride, const void* k_cache,

@@ -78,6 +78,7 @@ def _declare(lib: ctypes.CDLL) -> None:
             p, p, l, p, p, p, i, p, p, p, l, f, f, f, i, i, i, i, i, i, i, i, p,
         ],
         "lig_kv_scatter": [p, p, l, p, p, p, i, i, i, i, i, i, p],
+        "lig_temperature_scale_rows": [p, p, l, p, f, f, i, i, i, i, p],
     }
     for name, args in sigs.items():
         fn = getattr(lib, name)

@@ -331,3 +331,10 @@ def paged_attention_general(
             out[r:e] = o.to(out.dtype)
         r = e
     return out
+
+
+def temperature_scale_rows(q, positions, coef: float, every: float):
+    tau = query_temperature(positions, coef, every) if coef != 0.0 else 1.0
+    if coef == 0.0:
+        return q.contiguous().clone()
+    return (q.float() * tau[:, None]).to(q.dtype)
