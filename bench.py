@@ -95,7 +95,26 @@ def main() -> None:
         help="LoRA adapters on the SGMV path (default ON: BASELINE's metric "
         "is Llama-3-8B + 32 LoRAs; --no-lora for the base-model A/B)",
     )
+    ap.add_argument(
+        "--hybrid",
+        nargs="?",
+        const="engine,kernels",
+        default="",
+        metavar="PARTS",
+        help="instead of the serving workload: Tikarax beside Llama at equal "
+        "size (prefill/decode throughput through the engine, and the new "
+        "kernels beside their counterparts against the HBM roofline); "
+        "PARTS = engine, kernels or both (benchmarks/bench_hybrid.py)",
+    )
+    ap.add_argument("--hybrid-sizes", default="s,m")
     args = ap.parse_args()
+
+    if args.hybrid:
+        sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "benchmarks"))
+        import bench_hybrid
+
+        bench_hybrid.main(["--part", args.hybrid, "--sizes", args.hybrid_sizes])
+        return
 
     rank = int(os.environ.get("RANK", "0"))
     world = int(os.environ.get("WORLD_SIZE", "1"))

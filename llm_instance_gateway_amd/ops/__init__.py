@@ -417,6 +417,9 @@ def sigmoid_gate_mul(x: torch.Tensor, g: torch.Tensor) -> torch.Tensor:
     return torch_ref.sigmoid_gate_mul(x, g)
 
 
+MINGRU_CHUNKED_MIN_LEN = 128
+
+
 def mingru_scan(zxg, state, seg_start, seg_len, seg_slot, seg_fresh, max_len: int):
     """minGRU over the segments of a flat batch.  zxg [R, 3W] holds the gate
     and candidate pre-activations and the output gate; state [slots, W] fp32
@@ -430,9 +433,17 @@ def mingru_scan(zxg, state, seg_start, seg_len, seg_slot, seg_fresh, max_len: in
         out = torch.empty(R, W, dtype=zxg.dtype, device=zxg.device)
         es = zxg.element_size()
         base = zxg.data_ptr()
+        # long portions: three-pass scan over 32-step chunks (scratch holds
+        # each chunk's (decay product, local state) pair)
+        scratch = None
+        if max_len >= MINGRU_CHUNKED_MIN_LEN:
+            nchunk = (int(max_len) + 31) // 32
+            scratch = torch.empty(
+                2 * seg_start.shape[0] * nchunk * W, dtype=torch.float32, device=zxg.device
+            )
         _hl().lig_mingru_scan(
             _ptr(out), base, base + W * es, base + 2 * W * es, W3, _ptr(state),
-            _ptr(seg_start), _ptr(seg_len), _ptr(seg_slot), _ptr(seg_fresh),
+            _ptr(scratch), _ptr(seg_start), _ptr(seg_len), _ptr(seg_slot), _ptr(seg_fresh),
             seg_start.shape[0], int(max_len), W, _is_f32(zxg), _stream(),
         )
         return out

@@ -142,6 +142,63 @@ __global__ void kv_scatter_kernel(const T* __restrict__ k, const T* __restrict__
   }
 }
 
+// 16-byte chunks: every head row (D and Dv multiples of 8) is moved as whole
+// 8-element vectors, one thread per chunk.
+template <typename T>
+__global__ void kv_scatter_vec_kernel(const T* __restrict__ k, const T* __restrict__ v,
+                                      long src_stride, T* __restrict__ k_cache,
+                                      T* __restrict__ v_cache,
+                                      const int64_t* __restrict__ slot_mapping,
+                                      int R, int G, int D, int Dv, int BS) {
+  const int kc = G * D / 8, per_row = G * (D + Dv) / 8;
+  const long total = (long)R * per_row;
+  for (long idx = blockIdx.x * (long)blockDim.x + threadIdx.x; idx < total;
+       idx += gridDim.x * (long)blockDim.x) {
+    const long t = idx / per_row;
+    const int c = (int)(idx - t * per_row);
+    const int64_t slot = slot_mapping[t];
+    if (slot < 0) continue;
+    const long blk = slot / BS;
+    const int off = (int)(slot % BS);
+    float tmp[8];
+    if (c < kc) {
+      const int e = c * 8, g = e / D, d = e % D;
+      ld8(k + t * src_stride + e, tmp);
+      st8(k_cache + ((blk * G + g) * BS + off) * (long)D + d, tmp);
+    } else {
+      const int e = (c - kc) * 8, g = e / Dv, d = e % Dv;
+      ld8(v + t * src_stride + e, tmp);
+      st8(v_cache + ((blk * G + g) * BS + off) * (long)Dv + d, tmp);
+    }
+  }
+}
+
+template <typename T>
+__global__ void temperature_scale_rows_vec_kernel(T* __restrict__ out,
+                                                  const T* __restrict__ q, long q_stride,
+                                                  const int64_t* __restrict__ positions,
+                                                  float temp_coef, float temp_every,
+                                                  int temp_every_int, int C8, long n8) {
+  for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < n8;
+       i += gridDim.x * (long)blockDim.x) {
+    const long r = i / C8;
+    const int c = (int)(i - r * C8) * 8;
+    float tau = 1.f;
+    if (temp_coef != 0.f) {
+      const long pos = positions[r];
+      const float m = temp_every_int > 0
+                          ? (float)((pos + 1) / temp_every_int)
+                          : floorf((float)(pos + 1) / temp_every);
+      tau = 1.f + temp_coef * logf(m + 1.f);
+    }
+    float v[8];
+    ld8(q + r * q_stride + c, v);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) v[k] *= tau;
+    st8(out + i * 8, v);
+  }
+}
+
 // q_out[r, :] = q[r, :] * tau(position r): the query temperature applied
 // ahead of an attention kernel that takes one scalar scale.  Also packs the
 // strided q view (a column block of the fused projection) contiguously.
@@ -175,6 +232,22 @@ void lig_temperature_scale_rows(void* out, const void* q, long q_stride,
                                 int C, int is_f32, hipStream_t s) {
   const long n = (long)R * C;
   if (n <= 0) return;
+  if (C % 8 == 0 && q_stride % 8 == 0 && aligned16(out) && aligned16(q)) {
+    const long n8 = n / 8;
+    long g8 = (n8 + 255) / 256;
+    const int grid8 = (int)(g8 > 65535 ? 65535 : g8);
+    if (is_f32)
+      hipLaunchKernelGGL(temperature_scale_rows_vec_kernel<float>, dim3(grid8),
+                         dim3(256), 0, s, (float*)out, (const float*)q,
+                         q_stride, positions, temp_coef, temp_every,
+                         temp_every_int, C / 8, n8);
+    else
+      hipLaunchKernelGGL(temperature_scale_rows_vec_kernel<bf16s>, dim3(grid8),
+                         dim3(256), 0, s, (bf16s*)out, (const bf16s*)q,
+                         q_stride, positions, temp_coef, temp_every,
+                         temp_every_int, C / 8, n8);
+    return;
+  }
   long gl = (n + 255) / 256;
   const int grid = (int)(gl > 65535 ? 65535 : gl);
   if (is_f32)
@@ -219,6 +292,22 @@ void lig_kv_scatter(const void* k, const void* v, long src_stride,
                     hipStream_t s) {
   const long total = (long)R * G * (D + Dv);
   if (total <= 0) return;
+  if (D % 8 == 0 && Dv % 8 == 0 && src_stride % 8 == 0 && aligned16(k) &&
+      aligned16(v) && aligned16(k_cache) && aligned16(v_cache)) {
+    long g8 = (total / 8 + 255) / 256;
+    const int grid8 = (int)(g8 > 65535 ? 65535 : g8);
+    if (is_f32)
+      hipLaunchKernelGGL(kv_scatter_vec_kernel<float>, dim3(grid8), dim3(256),
+                         0, s, (const float*)k, (const float*)v, src_stride,
+                         (float*)k_cache, (float*)v_cache, slot_mapping, R, G,
+                         D, Dv, BS);
+    else
+      hipLaunchKernelGGL(kv_scatter_vec_kernel<bf16s>, dim3(grid8), dim3(256),
+                         0, s, (const bf16s*)k, (const bf16s*)v, src_stride,
+                         (bf16s*)k_cache, (bf16s*)v_cache, slot_mapping, R, G,
+                         D, Dv, BS);
+    return;
+  }
   long gl = (total + 255) / 256;
   const int grid = (int)(gl > 65535 ? 65535 : gl);
   if (is_f32)

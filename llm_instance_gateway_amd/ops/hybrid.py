@@ -73,7 +73,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "lig_post_add_pre_norm": [p, p, p, p, p, f, i, i, i, i, p],
         "lig_xielu": [p, p, f, f, l, i, p],
         "lig_sigmoid_gate_mul": [p, p, l, i, i, i, p],
-        "lig_mingru_scan": [p, p, p, p, l, p, p, p, p, p, i, i, i, i, p],
+        "lig_mingru_scan": [p, p, p, p, l, p, p, p, p, p, p, i, i, i, i, p],
         "lig_paged_attention_general": [
             p, p, l, p, p, p, i, p, p, p, l, f, f, f, i, i, i, i, i, i, i, i, p,
         ],

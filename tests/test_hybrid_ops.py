@@ -97,7 +97,7 @@ def _segs(device, start, length, slot, fresh):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("W", [1, 40, 130])
 def test_mingru_segments_state_and_slot_reuse(device, dtype, W):
-    lens = [1, 700 if W == 40 else 70, 9, 2]   # 700: the widest time split on the GPU
+    lens = [1, 70 if W == 130 else 700, 9, 2]   # 700: the chunked three-pass scan on the GPU
     R = sum(lens) + 3                          # trailing rows belong to no segment
     zxg = rnd(R, 3 * W, seed=10, dtype=dtype, s=1.5)
     state = torch.full((6, W), 123.0)          # stale garbage in every slot
