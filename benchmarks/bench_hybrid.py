@@ -56,10 +56,10 @@ def tikarax_config(name: str, z: dict) -> ModelConfig:
                 "type": "attention",
                 "mixer": {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"],
                           "vdim": z["dim"], "scale": 1.0 / math.sqrt(z["dim"]),
-                          "q_temp": {"coef": 0.5, "every": 64}},
+                          "q_temp": {"coef": 0.25, "every": 128}},
                 "mlp": mlp,
             })
-    return make_config(f"tikarax-{name}", z["vocab"], z["width"], layers, groups=2)
+    return make_config(f"tikarax-{name}", z["vocab"], z["width"], layers, groups=4)
 
 
 def llama_config(name: str, z: dict) -> ModelConfig:
@@ -197,7 +197,7 @@ def part_kernels(sizes) -> None:
             pos = torch.arange(T, device=dev, dtype=torch.int64)
             qv = proj[:, : hq * D]
             add("temperature_scale_rows", "rotary_embedding",
-                timeit(lambda: ops.temperature_scale_rows(qv, pos, 0.5, 64.0)), T * hq * D * 4)
+                timeit(lambda: ops.temperature_scale_rows(qv, pos, 0.25, 128.0)), T * hq * D * 4)
             qc, kc2 = qv.contiguous(), kk.clone()
             csc = ops.build_cos_sin_cache(D, T, 10000.0, dev).float()
             add("rotary_embedding", "temperature_scale_rows",
