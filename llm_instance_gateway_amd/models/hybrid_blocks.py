@@ -89,7 +89,9 @@ class GatedAttention(nn.Module):
         q, k, v = proj[:, :a], proj[:, a:b], proj[:, b:c]
         gate = proj[:, c:] if self.out_gate else None
         ops.kv_scatter(k, v, k_cache, v_cache, meta.slot_mapping)
-        if ops.mfma_attention_supported(proj.dtype, self.dim, self.vdim, proj.is_cuda):
+        if ops.mfma_attention_supported(
+            proj.dtype, self.dim, self.vdim, proj.is_cuda, self.heads // self.kv_heads
+        ):
             o = self._attend_mfma(q, gate, positions, k_cache, v_cache, meta)
         else:
             o = ops.paged_attention_general(

@@ -123,7 +123,8 @@ class TikaraxForCausalLM(nn.Module):
         self.needs_prefill_tiles = any(
             s.type == "attention"
             and ops.mfma_attention_supported(
-                dtype, s.mixer["dim"], s.mixer["vdim"], self.device_.type == "cuda"
+                dtype, s.mixer["dim"], s.mixer["vdim"], self.device_.type == "cuda",
+                s.mixer["heads"] // s.mixer["kv_heads"],
             )
             for s in cfg.layer_specs
         )
@@ -138,7 +139,7 @@ class TikaraxForCausalLM(nn.Module):
         for layer in self.layers:
             m = layer.mixer
             if isinstance(m, GatedAttention) and ops.mfma_attention_supported(
-                self.dtype_, m.dim, m.vdim, self.device_.type == "cuda"
+                self.dtype_, m.dim, m.vdim, self.device_.type == "cuda", m.heads // m.kv_heads
             ):
                 cand = (m.heads, m.kv_heads, m.dim)
                 if best is None or cand[0] * cand[2] > best[0] * best[2]:

@@ -519,14 +519,18 @@ def temperature_scale_rows(q, positions, coef: float, every: float) -> torch.Ten
     return torch_ref.temperature_scale_rows(q, positions, coef, every)
 
 
-def mfma_attention_supported(q_dtype, k_dim: int, v_dim: int, is_cuda: bool) -> bool:
+def mfma_attention_supported(
+    q_dtype, k_dim: int, v_dim: int, is_cuda: bool, group: int = 1
+) -> bool:
     """The MFMA flash-prefill / paged-decode kernels of the torch extension
-    serve bf16 caches with equal key and value head size 64 or 128."""
+    serve bf16 caches with equal key and value head size 64 or 128 and at
+    most 16 query heads per key/value head."""
     return (
         is_cuda
         and q_dtype == torch.bfloat16
         and k_dim == v_dim
         and k_dim in (64, 128)
+        and 1 <= group <= 16
         and os.environ.get("LIG_FORCE_TORCH_OPS") != "1"
         and os.environ.get("LIG_GENERAL_ATTENTION") != "1"
         and native_available()

@@ -21,7 +21,7 @@
 
 #define ATT_MAX_DV_PER_LANE 8  // Dv <= 512
 
-template <typename T>
+template <typename T, bool VEC>
 __global__ void paged_attention_general_kernel(
     T* __restrict__ out,  // [R, H * Dv]
     const T* __restrict__ q, long q_stride,
@@ -77,7 +77,16 @@ __global__ void paged_attention_general_kernel(
       const T* krow = k_cache + ((blk * G + g) * BS + off) * (long)D;
       voff = ((blk * G + g) * BS + off) * (long)Dv;
       float dot = 0.f;
-      for (int d = 0; d < D; ++d) dot += q_s[d] * ld(krow + d);
+      if (VEC) {  // D % 8 == 0 and 16-byte aligned rows: whole 8-element vectors
+        for (int d = 0; d < D; d += 8) {
+          float kv[8];
+          ld8(krow + d, kv);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) dot += q_s[d + i] * kv[i];
+        }
+      } else {
+        for (int d = 0; d < D; ++d) dot += q_s[d] * ld(krow + d);
+      }
       score = dot * sc;
     }
     const float m_new = fmaxf(m, wave_reduce_max(score));  // finite: key j0 is valid
@@ -270,20 +279,20 @@ void lig_paged_attention_general(
   if (R <= 0) return;
   dim3 grid(R, H), block(WAVE_SIZE);
   const size_t smem = (size_t)(((D + 1) & ~1) + WAVE_SIZE) * sizeof(float) + WAVE_SIZE * sizeof(long);
-  if (is_f32)
-    hipLaunchKernelGGL(paged_attention_general_kernel<float>, grid, block, smem,
-                       s, (float*)out, (const float*)q, q_stride,
-                       (const float*)k_cache, (const float*)v_cache,
-                       block_tables, max_blocks, tok_seq, positions,
-                       (const float*)gate, gate_stride, scale, temp_coef,
-                       temp_every, temp_every_int, H, G, D, Dv, BS);
-  else
-    hipLaunchKernelGGL(paged_attention_general_kernel<bf16s>, grid, block, smem,
-                       s, (bf16s*)out, (const bf16s*)q, q_stride,
-                       (const bf16s*)k_cache, (const bf16s*)v_cache,
-                       block_tables, max_blocks, tok_seq, positions,
-                       (const bf16s*)gate, gate_stride, scale, temp_coef,
-                       temp_every, temp_every_int, H, G, D, Dv, BS);
+  const bool vec = D % 8 == 0 && aligned16(k_cache);
+#define LIG_LAUNCH_ATT(T, VEC)                                                  \
+  hipLaunchKernelGGL((paged_attention_general_kernel<T, VEC>), grid, block,     \
+                     smem, s, (T*)out, (const T*)q, q_stride,                   \
+                     (const T*)k_cache, (const T*)v_cache, block_tables,        \
+                     max_blocks, tok_seq, positions, (const T*)gate,            \
+                     gate_stride, scale, temp_coef, temp_every, temp_every_int, \
+                     H, G, D, Dv, BS)
+  if (is_f32) {
+    if (vec) LIG_LAUNCH_ATT(float, true); else LIG_LAUNCH_ATT(float, false);
+  } else {
+    if (vec) LIG_LAUNCH_ATT(bf16s, true); else LIG_LAUNCH_ATT(bf16s, false);
+  }
+#undef LIG_LAUNCH_ATT
 }
 
 void lig_kv_scatter(const void* k, const void* v, long src_stride,

@@ -224,6 +224,32 @@ def test_attention_one_key_stands_out(device, bs):
 
 
 @pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_portion_rows_ignore_what_lies_past_them(device, dtype):
+    """A 40-row prompt portion at positions 100..139 of a sequence whose pages
+    still hold a dominating key at position 140 (left by an earlier, longer
+    user of the page): every row must return the value of the one standout
+    key far back (position 5), untouched by what lies past the portion."""
+    D, Dv, L = 24, 10, 160
+    k = rnd(L, D, seed=40, s=0.02)
+    v = rnd(L, Dv, seed=41)
+    q = rnd(1, D, seed=42)
+    q = (q / q.norm()).to(dtype).float()
+    k[5] = 30.0 * q[0]
+    k[140] = 60.0 * q[0]
+    kc, vc, bt = paged(device, dtype, k, v, 1, 16, 12, seed=9)
+    pos = list(range(100, 140))
+    R = len(pos)
+    out = ops.paged_attention_general(
+        q.repeat(R, 1).to(dtype).to(device), kc, vc, bt.view(1, -1).contiguous().to(device),
+        torch.zeros(R, dtype=torch.int32, device=device),
+        torch.tensor(pos, dtype=torch.int64, device=device), 1.0, 1,
+    )
+    v5 = v[5].to(dtype).double()
+    assert (out.double().cpu() - v5).abs().max().item() < (1e-3 if dtype == torch.float32 else 3e-2)
+
+
+@pytest.mark.parametrize("device", DEVICES)
 def test_query_temperature_on_both_sides_of_each_step(device):
     """tau(p) = 1 + c ln(floor((p+1)/e) + 1) changes between p = m*e - 2 and
     m*e - 1; two keys with different scores make the output depend on it."""

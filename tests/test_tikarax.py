@@ -237,8 +237,8 @@ def test_mixed_batch_equals_each_alone_and_pools_are_reused(model_a, device, dty
     plan = [
         [("a", 20), ("b", 3)],
         [("a", 1), ("b", 2), ("c", 30), ("d", 1)],           # b, d end: slots free
-        [("a", 16), ("c", 1), ("e", 7)],                      # e reuses a freed slot + pages
-        [("c", 19), ("e", 1), ("f", 2)],                      # a, c end
+        [("a", 16), ("e", 7)],                                # c sits this step out; e reuses a freed slot + pages
+        [("c", 20), ("e", 1), ("f", 2)],                      # a ended; c comes back and ends
         [("e", 15), ("f", 30)],
         [("f", 1)],
     ]
