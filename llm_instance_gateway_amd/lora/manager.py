@@ -116,6 +116,10 @@ class AdapterManager:
     ) -> None:
         self.engine = engine
         runner = engine.runner
+        if not getattr(runner.model, "supports_lora", True):
+            raise NotImplementedError(
+                f"{type(runner.model).__name__} has no LoRA hooks; it serves the base model only"
+            )
         self.device = runner.device
         self.dtype = runner.dtype
         mc = runner.config.model

@@ -95,6 +95,8 @@ class HybridLayer(nn.Module):
 class TikaraxForCausalLM(nn.Module):
     # the runner builds per-token sequence tables and per-sequence segments
     needs_seq_tables = True
+    # no adapter hooks in the mixers: base model only
+    supports_lora = False
     # decode-only steps replay hipGraphs (one-token segments, static tables)
     supports_decode_graphs = True
 

@@ -185,7 +185,8 @@ def _worker_main(
     torch.manual_seed(1234)  # same base weights on every engine of the pool
     eng = LLMEngine(cfg, device=device, tp=tp)
     mgr: Optional[AdapterManager] = None
-    if cfg.max_loras > 0:
+    # model families without LoRA hooks serve the base model only
+    if cfg.max_loras > 0 and getattr(eng.runner.model, "supports_lora", True):
         mgr = AdapterManager(eng, max_slots=cfg.max_loras, rank=lora_rank)
 
     seq_by_id: Dict[str, Any] = {}

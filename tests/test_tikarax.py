@@ -410,3 +410,32 @@ def test_decode_graphs_replay_like_eager(model_a, model_c, dtype, which):
     for seq, prompt in zip(seqs, prompts):
         assert seq.is_finished()
         assert_greedy_follows_oracle(cfg, W, prompt, seq.output_token_ids, margin)
+
+
+def test_served_through_the_pool_and_front_door(tmp_path):
+    """A model folder as the pool's base model: worker process, router, HTTP
+    front door, greedy completion from prompt token ids."""
+    from starlette.testclient import TestClient
+
+    from llm_instance_gateway_amd.api.types import InferenceModel
+    from llm_instance_gateway_amd.serving import EnginePool, build_app
+
+    cfg = dict(CFG_A, vocab=300)
+    W = make_checkpoint(cfg, 21)
+    path = write_model(tmp_path / "served", cfg, W)
+    pool = EnginePool(
+        path, devices=["cpu"],
+        engine_kwargs=dict(num_kv_blocks=64, max_num_seqs=4, max_num_batched_tokens=64, max_model_len=256),
+    )
+    pool.start()
+    try:
+        pool.datastore.store_model(InferenceModel(model_name="hybrid"))
+        client = TestClient(build_app(pool))
+        prompt = tokens_for(cfg, 23, 8)
+        r = client.post("/v1/completions", json={"model": "hybrid", "prompt": prompt, "max_tokens": 5})
+        assert r.status_code == 200, r.text
+        out = r.json()["choices"][0]["token_ids"]
+        assert len(out) == 5
+        assert_greedy_follows_oracle(cfg, W, prompt, out, margin=0.2)  # workers run bf16
+    finally:
+        pool.stop()
