@@ -208,6 +208,37 @@ def part_kernels(sizes) -> None:
             emb = torch.randn(z["vocab"], H, device=dev, dtype=bf)
             ids = torch.randint(0, z["vocab"], (T,), device=dev)
             add("embed_group_norm", "", timeit(lambda: ops.embed_group_norm(ids, emb, w, 1e-5, 2)), T * H * 6)
+            if T >= 1024:
+                # prompt attention: 8 fresh prompts of 1024 tokens, causal;
+                # flops = 2 (QK^T, PV) * 2 * sum over rows of keys seen * D * heads
+                L, S = 1024, T // 1024
+                nb_seq = L // bs
+                kcache = torch.randn(S * nb_seq + 1, hkv, bs, D, device=dev, dtype=bf)
+                vcache = torch.randn_like(kcache)
+                tables = torch.arange(S * nb_seq, dtype=torch.int32, device=dev).view(S, nb_seq)
+                qsl = i32([i * L for i in range(S + 1)])
+                ctxl = i32([L] * S)
+                tseq = i32([s_ for s_ in range(S) for _ in range(L // 64)])
+                tqs = i32([q0 for _ in range(S) for q0 in range(0, L, 64)])
+                tok_seq = i32([s_ for s_ in range(S) for _ in range(L)])
+                posq = torch.arange(L, device=dev, dtype=torch.int64).repeat(S)
+                flops = 4.0 * S * (L * (L + 1) / 2) * D * hq
+                sc = 1.0 / math.sqrt(D)
+
+                def addf(kernel, t):
+                    rows.append({"kernel": kernel, "like": "attention prefill", "us": round(t * 1e6, 1),
+                                 "TFLOP_per_s": round(flops / t / 1e12, 1)})
+
+                addf("paged_attention_prefill_tiles (temperature+gate fused)", timeit(
+                    lambda: ops.paged_attention_prefill_tiles(qv, kcache, vcache, tables, qsl, ctxl, tseq, tqs, sc, hq,
+                                                              gate=gv, temp_coef=0.25, temp_every=128.0), 10))
+                qh = qv.contiguous().view(T, hq, D)
+                addf("paged_attention_prefill (64/128 kernel of the Llama path)", timeit(
+                    lambda: ops.paged_attention_prefill(qh, kcache, vcache, tables, qsl, ctxl, sc,
+                                                        tile_seq=tseq, tile_qstart=tqs), 10))
+                addf("paged_attention_general (any-shape kernel)", timeit(
+                    lambda: ops.paged_attention_general(qv, kcache, vcache, tables, tok_seq, posq, sc, hq, gate=gv,
+                                                        temp_coef=0.25, temp_every=128.0), 3))
             print(json.dumps({"bench": "kernels", "size": name, "rows": T, "kernels": rows}), flush=True)
 
 

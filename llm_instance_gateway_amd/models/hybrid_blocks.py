@@ -93,6 +93,29 @@ class GatedAttention(nn.Module):
             proj.dtype, self.dim, self.vdim, proj.is_cuda, self.heads // self.kv_heads
         ):
             o = self._attend_mfma(q, gate, positions, k_cache, v_cache, meta)
+        elif (
+            meta.num_prefill_tokens > 0
+            and meta.prefill_tile_seq is not None
+            and ops.tiled_prefill_supported(proj.dtype, self.dim, self.vdim, proj.is_cuda)
+        ):
+            # prompt portions on MFMA tiles (temperature and gate fused), the
+            # step's single tokens (and pad rows) through the any-shape kernel
+            np_, rows = meta.num_prefill_tokens, proj.shape[0]
+            o = torch.empty(rows, self.heads * self.vdim, dtype=proj.dtype, device=proj.device)
+            ops.paged_attention_prefill_tiles(
+                q[:np_], k_cache, v_cache, meta.prefill_block_tables,
+                meta.prefill_query_start_locs, meta.prefill_context_lens,
+                meta.prefill_tile_seq, meta.prefill_tile_qstart, self.scale, self.heads,
+                gate=None if gate is None else gate[:np_], temp_coef=self.temp_coef,
+                temp_every=self.temp_every, out=o[:np_],
+            )
+            if rows > np_:
+                ops.paged_attention_general(
+                    q[np_:], k_cache, v_cache, meta.seq_block_tables, meta.tok_seq[np_:],
+                    positions[np_:], self.scale, self.heads,
+                    gate=None if gate is None else gate[np_:], temp_coef=self.temp_coef,
+                    temp_every=self.temp_every, out=o[np_:],
+                )
         else:
             o = ops.paged_attention_general(
                 q, k_cache, v_cache, meta.seq_block_tables, meta.tok_seq, positions,

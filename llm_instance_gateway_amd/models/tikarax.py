@@ -120,13 +120,17 @@ class TikaraxForCausalLM(nn.Module):
         self.layers = nn.ModuleList(
             [HybridLayer(s, H, device, dtype) for s in cfg.layer_specs]
         )
-        # any attention layer with bf16 and key size == value size in {64,128}
-        # runs the tiled MFMA prefill kernel and needs its 64-row query tiles
+        # attention layers whose prompt rows run an MFMA prefill kernel need
+        # the runner's 64-row query tiles
+        on_gpu = self.device_.type == "cuda"
         self.needs_prefill_tiles = any(
             s.type == "attention"
-            and ops.mfma_attention_supported(
-                dtype, s.mixer["dim"], s.mixer["vdim"], self.device_.type == "cuda",
-                s.mixer["heads"] // s.mixer["kv_heads"],
+            and (
+                ops.mfma_attention_supported(
+                    dtype, s.mixer["dim"], s.mixer["vdim"], on_gpu,
+                    s.mixer["heads"] // s.mixer["kv_heads"],
+                )
+                or ops.tiled_prefill_supported(dtype, s.mixer["dim"], s.mixer["vdim"], on_gpu)
             )
             for s in cfg.layer_specs
         )

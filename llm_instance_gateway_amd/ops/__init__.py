@@ -470,6 +470,7 @@ def kv_scatter(k, v, k_cache, v_cache, slot_mapping) -> None:
 def paged_attention_general(
     q, k_cache, v_cache, block_tables, tok_seq, positions, scale: float,
     num_heads: int, gate=None, temp_coef: float = 0.0, temp_every: float = 1.0,
+    out: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """Causal paged attention for any key/value head sizes; token r of the
     flat batch attends keys 0..positions[r] of sequence tok_seq[r].  Optional
@@ -485,7 +486,9 @@ def paged_attention_general(
         assert positions.dtype == torch.int64 and block_tables.is_contiguous()
         if gate is not None:
             assert gate.shape == (R, num_heads * Dv) and gate.stride(1) == 1
-        out = torch.empty(R, num_heads * Dv, dtype=q.dtype, device=q.device)
+        if out is None:
+            out = torch.empty(R, num_heads * Dv, dtype=q.dtype, device=q.device)
+        assert out.shape == (R, num_heads * Dv) and out.is_contiguous() and out.dtype == q.dtype
         ev = float(temp_every)
         ev_int = int(ev) if ev == int(ev) and ev >= 1 else 0
         _hl().lig_paged_attention_general(
@@ -496,10 +499,14 @@ def paged_attention_general(
             bs, _is_f32(q), _stream(),
         )
         return out
-    return torch_ref.paged_attention_general(
+    res = torch_ref.paged_attention_general(
         q, k_cache, v_cache, block_tables, tok_seq, positions, scale, num_heads,
         gate, temp_coef, temp_every,
     )
+    if out is not None:
+        out.copy_(res)
+        return out
+    return res
 
 
 def temperature_scale_rows(q, positions, coef: float, every: float) -> torch.Tensor:
@@ -535,3 +542,55 @@ def mfma_attention_supported(
         and os.environ.get("LIG_GENERAL_ATTENTION") != "1"
         and native_available()
     )
+
+
+def tiled_prefill_supported(q_dtype, k_dim: int, v_dim: int, is_cuda: bool) -> bool:
+    """The MFMA prefill kernel of the light library: bf16, key and value head
+    sizes independent, each a multiple of 8 and at most 128."""
+    return (
+        is_cuda
+        and q_dtype == torch.bfloat16
+        and k_dim % 8 == 0
+        and v_dim % 8 == 0
+        and 0 < k_dim <= 128
+        and 0 < v_dim <= 128
+        and os.environ.get("LIG_FORCE_TORCH_OPS") != "1"
+        and os.environ.get("LIG_GENERAL_ATTENTION") != "1"
+    )
+
+
+def paged_attention_prefill_tiles(
+    q, k_cache, v_cache, block_tables, query_start_locs, context_lens, tile_seq,
+    tile_qstart, scale: float, num_heads: int, gate=None, temp_coef: float = 0.0,
+    temp_every: float = 1.0, out: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """Prompt-partition attention on MFMA tiles for any head sizes the kernel
+    takes (`tiled_prefill_supported`): q [Tp, H*D] (strided view allowed) are
+    the rows of the step's prompt portions, laid out by query_start_locs;
+    context_lens count each sequence's tokens after this step; tile_seq /
+    tile_qstart name the 64-row query tiles.  Temperature and sigmoid gate are
+    fused.  GPU only."""
+    nb, G, bs, D = k_cache.shape
+    Dv = v_cache.shape[-1]
+    Tp = q.shape[0]
+    assert q.is_cuda and q.dtype == torch.bfloat16 and q.stride(1) == 1
+    assert q.shape[1] == num_heads * D
+    for t in (block_tables, query_start_locs, context_lens, tile_seq, tile_qstart):
+        assert t.dtype == torch.int32 and t.is_contiguous()
+    if gate is not None:
+        assert gate.shape == (Tp, num_heads * Dv) and gate.stride(1) == 1
+    if out is None:
+        out = torch.empty(Tp, num_heads * Dv, dtype=q.dtype, device=q.device)
+    assert out.shape == (Tp, num_heads * Dv) and out.is_contiguous()
+    ev = float(temp_every)
+    ev_int = int(ev) if ev == int(ev) and ev >= 1 else 0
+    rc = _hl().lig_paged_attention_prefill_tiles(
+        _ptr(out), _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(gate),
+        0 if gate is None else gate.stride(0), _ptr(tile_seq), _ptr(tile_qstart),
+        _ptr(query_start_locs), _ptr(context_lens), _ptr(block_tables), float(scale),
+        float(temp_coef), ev, ev_int, tile_seq.shape[0], num_heads, G, D, Dv, bs,
+        block_tables.shape[1], _stream(),
+    )
+    if rc != 0:
+        raise RuntimeError("paged_attention_prefill_tiles: shape or alignment not served")
+    return out

@@ -28,7 +28,10 @@ PKG = Path(__file__).resolve().parent.parent
 CSRC = Path(__file__).resolve().parent / "csrc"
 # Sources of the light library; setup.py leaves these out of the torch
 # extension.
-SOURCES = ["group_norm.hip", "xielu.hip", "mingru.hip", "attention_general.hip"]
+SOURCES = [
+    "group_norm.hip", "xielu.hip", "mingru.hip", "attention_general.hip",
+    "attention_prefill_tiles.hip",
+]
 SO_PATH = PKG / "_hybrid.so"
 
 _LIB: Optional[ctypes.CDLL] = None
@@ -84,6 +87,9 @@ def _declare(lib: ctypes.CDLL) -> None:
         fn = getattr(lib, name)
         fn.argtypes = args
         fn.restype = None
+    pt = lib.lig_paged_attention_prefill_tiles
+    pt.argtypes = [p, p, l, p, p, p, l, p, p, p, p, p, f, f, f, i, i, i, i, i, i, i, i, p]
+    pt.restype = ctypes.c_int
 
 
 def lib() -> ctypes.CDLL:

@@ -277,3 +277,61 @@ def test_query_temperature_on_both_sides_of_each_step(device):
     assert abs(o_query_temperature(5, c, e) - (1 + c * math.log(2))) < 1e-12
     # the step is visible in the outputs: p = 4 and p = 5 differ by more than rounding
     assert (out[1] - out[2]).abs().max().item() > 1e-2
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,G,D,Dv", [(4, 2, 8, 16), (6, 1, 48, 32), (2, 2, 80, 128), (3, 1, 24, 8), (2, 1, 128, 40), (1, 1, 64, 64)])
+@pytest.mark.parametrize("bs", [16, 8])
+def test_tiled_prefill_kernel(H, G, D, Dv, bs):
+    """MFMA prefill tiles for padded head sizes: three sequences in one launch
+    — a 100-row portion ending at position 149 (two query tiles, the second
+    partial, keys crossing 32-key tiles and pages), a fresh 5-token prompt, and
+    a fresh prompt of exactly one tile — with temperature and gate, from
+    strided q / gate views."""
+    device, dtype = "cuda:0", torch.bfloat16
+    assert ops.tiled_prefill_supported(dtype, D, Dv, True)
+    ctxs, ns = [150, 5, 64], [100, 5, 64]
+    nblk = sum((c + bs - 1) // bs for c in ctxs) + 2
+    g = torch.Generator().manual_seed(H * 100 + D)
+    perm = torch.randperm(nblk, generator=g).tolist()
+    kc = torch.full((nblk, G, bs, D), 7.0, dtype=dtype, device=device)
+    vc = torch.full((nblk, G, bs, Dv), -7.0, dtype=dtype, device=device)
+    maxb = max((c + bs - 1) // bs for c in ctxs)
+    tables = torch.zeros(len(ctxs), maxb, dtype=torch.int32)
+    ks, vs, at = [], [], 0
+    for s, c in enumerate(ctxs):
+        nb = (c + bs - 1) // bs
+        blocks = perm[at : at + nb]
+        at += nb
+        tables[s, :nb] = torch.tensor(blocks, dtype=torch.int32)
+        k = rnd(c, G * D, seed=50 + s, s=0.6).to(dtype)
+        v = rnd(c, G * Dv, seed=60 + s).to(dtype)
+        pos = torch.arange(c)
+        slots = (torch.tensor(blocks)[pos // bs] * bs + pos % bs).to(torch.int64).to(device)
+        fused = torch.cat([k, v], dim=1).to(device)
+        ops.kv_scatter(fused[:, : G * D], fused[:, G * D :], kc, vc, slots)
+        ks.append(k.to(F64))
+        vs.append(v.to(F64))
+    Tp = sum(ns)
+    q = rnd(Tp, H * D, seed=70).to(dtype)
+    gate = rnd(Tp, H * Dv, seed=71).to(dtype)
+    fused = torch.cat([q, torch.zeros(Tp, 8, dtype=dtype), gate], dim=1).to(device)
+    qsl = [0]
+    for n in ns:
+        qsl.append(qsl[-1] + n)
+    ts, tq = [], []
+    for s, n in enumerate(ns):
+        for q0 in range(0, n, 64):
+            ts.append(s)
+            tq.append(q0)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=device)
+    scale, coef, every = 0.9 / math.sqrt(D), 0.7, 16
+    out = ops.paged_attention_prefill_tiles(
+        fused[:, : H * D], kc, vc, tables.to(device), i32(qsl), i32(ctxs), i32(ts), i32(tq),
+        scale, H, gate=fused[:, H * D + 8 :], temp_coef=coef, temp_every=every,
+    )
+    for s, (c, n) in enumerate(zip(ctxs, ns)):
+        rows = slice(qsl[s], qsl[s + 1])
+        want = o_attention(q[rows].to(F64), ks[s], vs[s], H, G, scale, coef, every,
+                           gate=gate[rows].to(F64), start=c - n)
+        close(out[rows], want, dtype)
