@@ -99,24 +99,31 @@ def engine_run(mc: ModelConfig, n_seqs: int, prompt_len: int, decode_steps: int)
     fill(4)
     prefill_phase()
     eng.generate_all()
-    # timed
-    fill(decode_steps + 1)
-    t_prefill = prefill_phase()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    steps = 0
-    while eng.has_work():
-        eng.step()
-        steps += 1
-    torch.cuda.synchronize()
-    t_decode = time.perf_counter() - t0
-    eng.collect_finished()
+    # timed: median of three rounds (a round = all prompts prefilled, then
+    # every sequence decoded to its end)
+    t_pre, t_dec, n_steps = [], [], []
+    for _ in range(3):
+        fill(decode_steps + 1)
+        t_pre.append(prefill_phase())
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        steps = 0
+        while eng.has_work():
+            eng.step()
+            steps += 1
+        torch.cuda.synchronize()
+        t_dec.append((time.perf_counter() - t0) / max(steps, 1))
+        n_steps.append(steps)
+        eng.collect_finished()
     del eng
     torch.cuda.empty_cache()
+    t_prefill = sorted(t_pre)[1]
+    t_step = sorted(t_dec)[1]
     return {
         "prefill_tok_per_s": round(n_seqs * prompt_len / t_prefill, 1),
-        "decode_tok_per_s": round(n_seqs * steps / t_decode, 1),
-        "decode_ms_per_step": round(t_decode / max(steps, 1) * 1e3, 3),
+        "decode_tok_per_s": round(n_seqs / t_step, 1),
+        "decode_ms_per_step": round(t_step * 1e3, 3),
+        "prefill_s_rounds": [round(t, 4) for t in t_pre],
     }
 
 
@@ -239,6 +246,25 @@ def part_kernels(sizes) -> None:
                 addf("paged_attention_general (any-shape kernel)", timeit(
                     lambda: ops.paged_attention_general(qv, kcache, vcache, tables, tok_seq, posq, sc, hq, gate=gv,
                                                         temp_coef=0.25, temp_every=128.0), 3))
+            else:
+                # decode attention: T sequences with 1024 cached tokens each;
+                # bytes = K and V of every sequence once
+                L = 1024
+                nb_seq = L // bs
+                kcache = torch.randn(T * nb_seq + 1, hkv, bs, D, device=dev, dtype=bf)
+                vcache = torch.randn_like(kcache)
+                tables = torch.arange(T * nb_seq, dtype=torch.int32, device=dev).view(T, nb_seq)
+                ctxl = i32([L] * T)
+                posd = torch.full((T,), L - 1, device=dev, dtype=torch.int64)
+                tok_seq = i32(list(range(T)))
+                kvbytes = T * L * hkv * D * 2 * 2
+                sc = 1.0 / math.sqrt(D)
+                qh = qv.contiguous().view(T, hq, D)
+                add("paged_attention_general (decode rows, gate+temperature fused)", "",
+                    timeit(lambda: ops.paged_attention_general(qv, kcache, vcache, tables, tok_seq, posd, sc, hq,
+                                                               gate=gv, temp_coef=0.25, temp_every=128.0), 10), kvbytes)
+                add("paged_attention_decode (64/128 kernel of the Llama path)", "paged_attention_general",
+                    timeit(lambda: ops.paged_attention_decode(qh, kcache, vcache, tables, ctxl, sc, max_ctx=L), 10), kvbytes)
             print(json.dumps({"bench": "kernels", "size": name, "rows": T, "kernels": rows}), flush=True)
 
 
