@@ -334,7 +334,7 @@ def paged_attention_general(
 
 
 def temperature_scale_rows(q, positions, coef: float, every: float):
-    tau = query_temperature(positions, coef, every) if coef != 0.0 else 1.0
     if coef == 0.0:
         return q.contiguous().clone()
+    tau = query_temperature(positions, coef, every)
     return (q.float() * tau[:, None]).to(q.dtype)

@@ -245,7 +245,6 @@ def test_mixed_batch_equals_each_alone_and_pools_are_reused(model_a, device, dty
     eng = make_engine(model_a[0], device, dtype, blocks=9, block_size=16, seqs=4)
     at = {k: 0 for k in toks}
     got = {k: [] for k in toks}
-    slots_seen = {}
     for step in plan:
         entries, end = [], []
         for rid, n in step:
@@ -253,12 +252,9 @@ def test_mixed_batch_equals_each_alone_and_pools_are_reused(model_a, device, dty
             at[rid] += n
             if at[rid] == lens[rid]:
                 end.append(rid)
-        live_before = dict(eng._replay_live)
         res = eng.replay_step(entries, end)
         for rid, _ in step:
             got[rid].append(res[rid].float().cpu())
-        for rid, seq in {**live_before, **eng._replay_live}.items():
-            slots_seen.setdefault(rid, set())
     assert all(at[k] == lens[k] for k in lens)
     bm = eng.scheduler.block_manager
     assert bm.num_free_blocks == 9 and bm.num_free_state_slots == 4
