@@ -98,27 +98,34 @@ class ModelRunner:
             if mc.has_recurrent_state:
                 self.num_state_slots = config.num_state_slots or config.max_num_seqs
             self.kv_caches = []
-            for spec in self.model.cache_specs():
+
+            def make(spec) -> tuple:
                 if spec["kind"] == "kv":
                     g = spec["kv_heads"]
-                    self.kv_caches.append(
-                        (
-                            torch.zeros((nblk, g, config.block_size, spec["k_dim"]), dtype=dtype, device=self.device),
-                            torch.zeros((nblk, g, config.block_size, spec["v_dim"]), dtype=dtype, device=self.device),
-                        )
+                    return (
+                        torch.zeros((nblk, g, config.block_size, spec["k_dim"]), dtype=dtype, device=self.device),
+                        torch.zeros((nblk, g, config.block_size, spec["v_dim"]), dtype=dtype, device=self.device),
                     )
-                elif spec["kind"] == "state":
-                    self.kv_caches.append(
-                        (
-                            torch.zeros(
-                                (self.num_state_slots + 1, spec["width"]),
-                                dtype=torch.float32,
-                                device=self.device,
-                            ),
-                        )
+                if spec["kind"] == "latent":
+                    # one shared row per token: keys and values are read from it
+                    return (
+                        torch.zeros((nblk, 1, config.block_size, spec["row"]), dtype=dtype, device=self.device),
                     )
-                else:
-                    raise ValueError(f"unknown cache kind {spec['kind']!r}")
+                if spec["kind"] == "state":
+                    return (
+                        torch.zeros(
+                            (self.num_state_slots + 1, spec["width"]),
+                            dtype=torch.float32,
+                            device=self.device,
+                        ),
+                    )
+                raise ValueError(f"unknown cache kind {spec['kind']!r}")
+
+            # an entry is one spec, or a list of specs whose tensors are
+            # handed to the layer together (paged rows plus a state row)
+            for spec in self.model.cache_specs():
+                parts = spec if isinstance(spec, (list, tuple)) else [spec]
+                self.kv_caches.append(tuple(t for p in parts for t in make(p)))
         else:
             shape = (nblk, kvh, config.block_size, mc.head_dim)
             self.kv_caches: List[Tuple[torch.Tensor, torch.Tensor]] = [

@@ -11,7 +11,7 @@ initialised randomly and the benchmark is synthetic-data.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Any, Dict, List, Optional
+from typing import Any, Dict, List, Optional, Tuple
 
 
 @dataclass
@@ -19,11 +19,15 @@ class LayerSpec:
     """One layer of a heterogeneous (hybrid) stack: which sequence mixer it
     has ('attention' keeps paged K/V, 'mingru' keeps a recurrent state
     vector), the mixer's sizes and constants, and its feed-forward (None for
-    a layer without one)."""
+    a layer without one).  'latent_attention' keeps one paged row per token
+    (the normalised key/value latent followed by the shared rotated key
+    part).  `shift` says the mixer's input is blended with the previous
+    token's, which costs one fp32 row of model width per sequence."""
 
     type: str
     mixer: Dict[str, Any] = field(default_factory=dict)
     mlp: Optional[Dict[str, Any]] = None
+    shift: bool = False
 
 
 @dataclass
@@ -56,12 +60,26 @@ class ModelConfig:
     # a row into (1 = ordinary RMS norm).
     layer_specs: Optional[List[LayerSpec]] = None
     norm_groups: int = 1
+    # Weight-shared loop over a span of layers: (start, stop, times) runs
+    # layers start..stop-1 `times` times in a row; every run of a layer has
+    # its own cache and state.  None = every layer runs once.
+    layer_loop: Optional[Tuple[int, int, int]] = None
     # Folder with config.json + model.safetensors ("" = random init).
     weights_path: str = ""
 
     @property
     def is_moe(self) -> bool:
+        if self.layer_specs is not None:
+            return any(s.mlp is not None and s.mlp.get("kind") == "moe" for s in self.layer_specs)
         return self.num_experts > 0
+
+    def layer_run_order(self) -> List[int]:
+        """Layer indices in the order they execute (a looped span repeats)."""
+        n = len(self.layer_specs) if self.layer_specs is not None else self.num_layers
+        if self.layer_loop is None:
+            return list(range(n))
+        a, b, times = self.layer_loop
+        return list(range(a)) + list(range(a, b)) * times + list(range(b, n))
 
     @property
     def kv_bytes_per_token_per_layer(self) -> int:
@@ -73,17 +91,27 @@ class ModelConfig:
         paged cache (recurrent layers keep none)."""
         if self.layer_specs is None:
             return self.num_layers * 2 * (self.num_kv_heads // tp_size) * self.head_dim
-        return sum(
-            (s.mixer["kv_heads"] // tp_size) * (s.mixer["dim"] + s.mixer["vdim"])
-            for s in self.layer_specs
-            if s.type == "attention"
-        )
+        total = 0
+        for i in self.layer_run_order():
+            s = self.layer_specs[i]
+            if s.type == "attention":
+                total += (s.mixer["kv_heads"] // tp_size) * (s.mixer["dim"] + s.mixer["vdim"])
+            elif s.type == "latent_attention":
+                total += s.mixer["kv_rank"] + s.mixer["rot_dim"]
+        return total
 
     def state_elems_per_seq(self) -> int:
         """fp32 recurrent-state elements one live sequence occupies."""
         if self.layer_specs is None:
             return 0
-        return sum(s.mixer["width"] for s in self.layer_specs if s.type == "mingru")
+        total = 0
+        for i in self.layer_run_order():
+            s = self.layer_specs[i]
+            if s.type == "mingru":
+                total += s.mixer["width"]
+            if s.shift:
+                total += self.hidden_size
+        return total
 
     @property
     def has_recurrent_state(self) -> bool:

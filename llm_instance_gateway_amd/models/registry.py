@@ -44,7 +44,20 @@ def _tikarax_config(raw: dict, path: str) -> ModelConfig:
     return config_from_json(raw, path)
 
 
+def _lopovik_factory(cfg, device, dtype, tp):
+    from .lopovik import LopovikForCausalLM
+
+    return LopovikForCausalLM(cfg, device=device, dtype=dtype, tp=tp)
+
+
+def _lopovik_config(raw: dict, path: str) -> ModelConfig:
+    from .lopovik import config_from_json
+
+    return config_from_json(raw, path)
+
+
 register_architecture("llama", None, _llama_factory)
+register_architecture("lopovik", _lopovik_config, _lopovik_factory)
 register_architecture("tikarax", _tikarax_config, _tikarax_factory)
 
 

@@ -467,18 +467,33 @@ def kv_scatter(k, v, k_cache, v_cache, slot_mapping) -> None:
     torch_ref.kv_scatter(k, v, k_cache, v_cache, slot_mapping)
 
 
+def _value_row_stride(v_cache: torch.Tensor) -> int:
+    """Entries between consecutive value rows of a [blocks, G, BS, Dv] cache
+    (or of a view of the leading Dv entries of a wider cache's rows)."""
+    nb, G, bs, Dv = v_cache.shape
+    v_row = v_cache.stride(2)
+    assert v_cache.stride(3) == 1 and v_row >= Dv
+    assert v_cache.stride(1) == bs * v_row and v_cache.stride(0) == G * bs * v_row
+    return v_row
+
+
 def paged_attention_general(
     q, k_cache, v_cache, block_tables, tok_seq, positions, scale: float,
     num_heads: int, gate=None, temp_coef: float = 0.0, temp_every: float = 1.0,
-    out: Optional[torch.Tensor] = None,
+    out: Optional[torch.Tensor] = None, sink: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """Causal paged attention for any key/value head sizes; token r of the
     flat batch attends keys 0..positions[r] of sequence tok_seq[r].  Optional
-    query temperature 1 + coef*ln(floor((p+1)/every)+1) and sigmoid output
-    gate.  q/gate may be column-block views with a row stride."""
+    query temperature 1 + coef*ln(floor((p+1)/every)+1), sigmoid output gate
+    and per-head softmax sink (fp32 [heads]: exp(sink) joins the denominator).
+    q/gate may be column-block views with a row stride; v_cache may be a view
+    of the leading entries of k_cache's rows (a latent cache)."""
     if _use_hybrid(q):
         nb, G, bs, D = k_cache.shape
         Dv = v_cache.shape[-1]
+        v_row = _value_row_stride(v_cache)
+        if sink is not None:
+            assert sink.dtype == torch.float32 and sink.shape == (num_heads,) and sink.is_contiguous()
         R = q.shape[0]
         assert q.shape[1] == num_heads * D and q.stride(1) == 1
         assert num_heads % G == 0 and Dv <= 512
@@ -495,13 +510,13 @@ def paged_attention_general(
             _ptr(out), _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache),
             _ptr(block_tables), block_tables.shape[1], _ptr(tok_seq),
             _ptr(positions), _ptr(gate), 0 if gate is None else gate.stride(0),
-            float(scale), float(temp_coef), ev, ev_int, R, num_heads, G, D, Dv,
-            bs, _is_f32(q), _stream(),
+            _ptr(sink), float(scale), float(temp_coef), ev, ev_int, R, num_heads,
+            G, D, Dv, v_row, bs, _is_f32(q), _stream(),
         )
         return out
     res = torch_ref.paged_attention_general(
         q, k_cache, v_cache, block_tables, tok_seq, positions, scale, num_heads,
-        gate, temp_coef, temp_every,
+        gate, temp_coef, temp_every, sink,
     )
     if out is not None:
         out.copy_(res)
@@ -563,15 +578,20 @@ def paged_attention_prefill_tiles(
     q, k_cache, v_cache, block_tables, query_start_locs, context_lens, tile_seq,
     tile_qstart, scale: float, num_heads: int, gate=None, temp_coef: float = 0.0,
     temp_every: float = 1.0, out: Optional[torch.Tensor] = None,
+    sink: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """Prompt-partition attention on MFMA tiles for any head sizes the kernel
     takes (`tiled_prefill_supported`): q [Tp, H*D] (strided view allowed) are
     the rows of the step's prompt portions, laid out by query_start_locs;
     context_lens count each sequence's tokens after this step; tile_seq /
-    tile_qstart name the 64-row query tiles.  Temperature and sigmoid gate are
-    fused.  GPU only."""
+    tile_qstart name the 64-row query tiles.  Temperature, sigmoid gate and
+    softmax sink are fused; v_cache may view the head of k_cache's rows.  GPU
+    only."""
     nb, G, bs, D = k_cache.shape
     Dv = v_cache.shape[-1]
+    v_row = _value_row_stride(v_cache)
+    if sink is not None:
+        assert sink.dtype == torch.float32 and sink.shape == (num_heads,) and sink.is_contiguous()
     Tp = q.shape[0]
     assert q.is_cuda and q.dtype == torch.bfloat16 and q.stride(1) == 1
     assert q.shape[1] == num_heads * D
@@ -586,11 +606,144 @@ def paged_attention_prefill_tiles(
     ev_int = int(ev) if ev == int(ev) and ev >= 1 else 0
     rc = _hl().lig_paged_attention_prefill_tiles(
         _ptr(out), _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(gate),
-        0 if gate is None else gate.stride(0), _ptr(tile_seq), _ptr(tile_qstart),
-        _ptr(query_start_locs), _ptr(context_lens), _ptr(block_tables), float(scale),
-        float(temp_coef), ev, ev_int, tile_seq.shape[0], num_heads, G, D, Dv, bs,
-        block_tables.shape[1], _stream(),
+        0 if gate is None else gate.stride(0), _ptr(sink), _ptr(tile_seq),
+        _ptr(tile_qstart), _ptr(query_start_locs), _ptr(context_lens),
+        _ptr(block_tables), float(scale), float(temp_coef), ev, ev_int,
+        tile_seq.shape[0], num_heads, G, D, Dv, v_row, bs, block_tables.shape[1],
+        _stream(),
     )
     if rc != 0:
         raise RuntimeError("paged_attention_prefill_tiles: shape or alignment not served")
     return out
+
+
+# -- token shift, latent attention, routed feed-forward -------------------------
+
+def residual_add(x: torch.Tensor, a: torch.Tensor, b: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x += a (+ b) in place; x is the fp32 residual, a and b branch outputs."""
+    assert x.dtype == torch.float32 and a.shape == x.shape and (b is None or b.shape == x.shape)
+    if _use_hybrid(x):
+        assert x.is_contiguous() and a.is_contiguous() and (b is None or b.is_contiguous())
+        assert b is None or b.dtype == a.dtype
+        _hl().lig_residual_add(_ptr(x), _ptr(a), _ptr(b), x.numel(), _is_f32(a), _stream())
+        return x
+    return torch_ref.residual_add(x, a, b)
+
+
+def offset_rms_norm(x: torch.Tensor, w: torch.Tensor, eps: float) -> torch.Tensor:
+    """fp32 rows -> x / rms(x) * (1 + w) in w's dtype."""
+    assert x.dtype == torch.float32
+    if _use_hybrid(x):
+        R, H = x.shape
+        assert x.is_contiguous()
+        out = torch.empty(R, H, dtype=w.dtype, device=x.device)
+        _hl().lig_offset_rms_norm(_ptr(out), _ptr(x), _ptr(w), float(eps), R, H, _is_f32(w), _stream())
+        return out
+    return torch_ref.offset_rms_norm(x, w, eps, w.dtype)
+
+
+def offset_norm_shift(
+    x, w_mix, w_ff, mu, state, tok_seq, seg_start, seg_len, seg_slot, seg_fresh, eps: float
+):
+    """Both input norms of a parallel layer from one pass over the fp32
+    residual x [R, H] (weights stored as offsets from one), with the mixer
+    branch blended with the previous token's, h + (h_prev - h) * mu.  `state`
+    [slots, H] fp32 carries each sequence's last unblended h between steps
+    and is updated in place.  w_ff None: no feed-forward branch.  Returns
+    (mixer input, feed-forward input or None) in w_mix's dtype; rows of no
+    segment are zero."""
+    assert x.dtype == torch.float32 and state.dtype == torch.float32
+    if _use_hybrid(x):
+        R, H = x.shape
+        assert x.is_contiguous() and state.shape[1] == H and state.is_contiguous()
+        hm = torch.empty(R, H, dtype=w_mix.dtype, device=x.device)
+        hf = None if w_ff is None else torch.empty_like(hm)
+        _hl().lig_offset_norm_shift(
+            _ptr(hm), _ptr(hf), _ptr(x), _ptr(w_mix), _ptr(w_ff), _ptr(mu), _ptr(state),
+            _ptr(tok_seq), _ptr(seg_start), _ptr(seg_len), _ptr(seg_slot), _ptr(seg_fresh),
+            float(eps), R, H, _is_f32(w_mix), _stream(),
+        )
+        return hm, hf
+    return torch_ref.offset_norm_shift(
+        x, w_mix, w_ff, mu, state, tok_seq, seg_start, seg_len, seg_slot, seg_fresh, eps,
+        w_mix.dtype,
+    )
+
+
+rotary_inv_freq = torch_ref.rotary_inv_freq
+
+
+def latent_kv_prep(
+    proj, q_rank: int, kv_rank: int, rot_dim: int, w_q, w_kv, eps: float, inv_freq,
+    positions, slot_mapping, cache,
+) -> torch.Tensor:
+    """Per row of the fused projection [query latent | key/value latent |
+    shared rotated key part | ...]: returns the RMS-normed query latent and
+    writes [normed key/value latent | rotated key part] into the paged latent
+    cache [blocks, 1, block_size, kv_rank + rot_dim] at slot_mapping."""
+    if _use_hybrid(proj):
+        R = proj.shape[0]
+        assert proj.stride(1) == 1 and proj.shape[1] >= q_rank + kv_rank + rot_dim
+        assert cache.is_contiguous() and cache.shape[1] == 1 and cache.shape[3] == kv_rank + rot_dim
+        assert cache.dtype == proj.dtype and inv_freq.dtype == torch.float32
+        assert positions.dtype == torch.int64 and slot_mapping.dtype == torch.int64
+        assert 2 * inv_freq.shape[0] <= rot_dim
+        cq = torch.empty(R, q_rank, dtype=proj.dtype, device=proj.device)
+        _hl().lig_latent_kv_prep(
+            _ptr(cq), _ptr(proj), proj.stride(0), _ptr(w_q), _ptr(w_kv), _ptr(inv_freq),
+            inv_freq.shape[0], _ptr(positions), _ptr(slot_mapping), _ptr(cache), float(eps),
+            R, q_rank, kv_rank, rot_dim, _is_f32(proj), _stream(),
+        )
+        return cq
+    return torch_ref.latent_kv_prep(
+        proj, q_rank, kv_rank, rot_dim, w_q, w_kv, eps, inv_freq, positions, slot_mapping, cache
+    )
+
+
+def rotate_pack_queries(q, heads: int, dim: int, rot_dim: int, inv_freq, positions, out, lead: int):
+    """out[r, h, lead:] = interleaved rotation of q[r, h, dim:dim+rot_dim];
+    q [R, heads*(dim+rot_dim)] contiguous, out [R, heads, lead+rot_dim]."""
+    if _use_hybrid(q):
+        R = q.shape[0]
+        assert q.is_contiguous() and out.is_contiguous() and out.dtype == q.dtype
+        assert out.shape == (R, heads, lead + rot_dim) and positions.dtype == torch.int64
+        _hl().lig_rotate_pack_queries(
+            _ptr(out), _ptr(q), _ptr(inv_freq), inv_freq.shape[0], _ptr(positions), R,
+            heads, dim, rot_dim, lead, _is_f32(q), _stream(),
+        )
+        return out
+    return torch_ref.rotate_pack_queries(q, heads, dim, rot_dim, inv_freq, positions, out, lead)
+
+
+def relu_squared(x: torch.Tensor) -> torch.Tensor:
+    if _use_hybrid(x):
+        assert x.is_contiguous()
+        out = torch.empty_like(x)
+        _hl().lig_relu_squared(_ptr(out), _ptr(x), x.numel(), _is_f32(x), _stream())
+        return out
+    return torch_ref.relu_squared(x)
+
+
+def silu_mul(x: torch.Tensor) -> torch.Tensor:
+    """[rows, 2F] fused (gate | up) -> silu(gate) * up [rows, F]; the light
+    library's own kernel (bf16 or fp32 storage)."""
+    if _use_hybrid(x):
+        assert x.is_contiguous() and x.dim() == 2 and x.shape[1] % 2 == 0
+        F_ = x.shape[1] // 2
+        out = torch.empty(x.shape[0], F_, dtype=x.dtype, device=x.device)
+        _hl().lig_silu_mul(_ptr(out), _ptr(x), x.shape[0], F_, _is_f32(x), _stream())
+        return out
+    return torch_ref.silu_and_mul(x)
+
+
+def scale_gather_rows(x: torch.Tensor, idx: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """out[i] = w[i] * x[idx[i]]; idx int64 (negative: zero row), w fp32."""
+    if _use_hybrid(x):
+        assert x.is_contiguous() and idx.dtype == torch.int64 and w.dtype == torch.float32
+        assert idx.is_contiguous() and w.is_contiguous() and idx.shape == w.shape
+        out = torch.empty(idx.shape[0], x.shape[1], dtype=x.dtype, device=x.device)
+        _hl().lig_scale_gather_rows(
+            _ptr(out), _ptr(x), _ptr(idx), _ptr(w), idx.shape[0], x.shape[1], _is_f32(x), _stream()
+        )
+        return out
+    return torch_ref.scale_gather_rows(x, idx, w)

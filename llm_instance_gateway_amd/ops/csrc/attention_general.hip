@@ -15,7 +15,13 @@
 // multiplies the score (same as scaling q), and an optional output gate
 // multiplies the result element-wise by sigmoid(gate) before it is stored.
 //
-// Cache layout: K [blocks, G, BS, D], V [blocks, G, BS, Dv].
+// An optional per-head sink adds exp(sink_h) to the softmax denominator: a
+// key with that (unscaled) score and no value, counted once per row.  The
+// running max starts at the sink and the running sum at one.
+//
+// Cache layout: K [blocks, G, BS, D], V [blocks, G, BS, v_row] of which the
+// first Dv entries of a row are the value (v_row == Dv for a cache of its
+// own; a latent cache passes the key rows themselves, v_row == D).
 
 #include "elem_types.h"
 
@@ -29,8 +35,9 @@ __global__ void paged_attention_general_kernel(
     const int* __restrict__ block_tables, int max_blocks,
     const int* __restrict__ tok_seq,        // [R], -1 = padding row
     const int64_t* __restrict__ positions,  // [R]
-    const T* __restrict__ gate, long gate_stride, float scale, float temp_coef,
-    float temp_every, int temp_every_int, int H, int G, int D, int Dv, int BS) {
+    const T* __restrict__ gate, long gate_stride, const float* __restrict__ sink,
+    float scale, float temp_coef, float temp_every, int temp_every_int, int H,
+    int G, int D, int Dv, int v_row, int BS) {
   extern __shared__ __align__(16) float smem[];
   float* q_s = smem;                       // [D], padded to an even count
   float* p_s = smem + ((D + 1) & ~1);      // [64]
@@ -62,6 +69,10 @@ __global__ void paged_attention_general_kernel(
   __syncthreads();
 
   float m = -INFINITY, l = 0.f;
+  if (sink != nullptr) {
+    m = sink[h];
+    l = 1.f;
+  }
   float acc[ATT_MAX_DV_PER_LANE];
 #pragma unroll
   for (int i = 0; i < ATT_MAX_DV_PER_LANE; ++i) acc[i] = 0.f;
@@ -75,7 +86,7 @@ __global__ void paged_attention_general_kernel(
       const long blk = bt[j / BS];
       const int off = j % BS;
       const T* krow = k_cache + ((blk * G + g) * BS + off) * (long)D;
-      voff = ((blk * G + g) * BS + off) * (long)Dv;
+      voff = ((blk * G + g) * BS + off) * (long)v_row;
       float dot = 0.f;
       if (VEC) {  // D % 8 == 0 and 16-byte aligned rows: whole 8-element vectors
         for (int d = 0; d < D; d += 8) {
@@ -273,9 +284,9 @@ void lig_paged_attention_general(
     void* out, const void* q, long q_stride, const void* k_cache,
     const void* v_cache, const int* block_tables, int max_blocks,
     const int* tok_seq, const int64_t* positions, const void* gate,
-    long gate_stride, float scale, float temp_coef, float temp_every,
-    int temp_every_int, int R, int H, int G, int D, int Dv, int BS, int is_f32,
-    hipStream_t s) {
+    long gate_stride, const float* sink, float scale, float temp_coef,
+    float temp_every, int temp_every_int, int R, int H, int G, int D, int Dv,
+    int v_row, int BS, int is_f32, hipStream_t s) {
   if (R <= 0) return;
   dim3 grid(R, H), block(WAVE_SIZE);
   const size_t smem = (size_t)(((D + 1) & ~1) + WAVE_SIZE) * sizeof(float) + WAVE_SIZE * sizeof(long);
@@ -285,8 +296,8 @@ void lig_paged_attention_general(
                      smem, s, (T*)out, (const T*)q, q_stride,                   \
                      (const T*)k_cache, (const T*)v_cache, block_tables,        \
                      max_blocks, tok_seq, positions, (const T*)gate,            \
-                     gate_stride, scale, temp_coef, temp_every, temp_every_int, \
-                     H, G, D, Dv, BS)
+                     gate_stride, sink, scale, temp_coef, temp_every,           \
+                     temp_every_int, H, G, D, Dv, v_row, BS)
   if (is_f32) {
     if (vec) LIG_LAUNCH_ATT(float, true); else LIG_LAUNCH_ATT(float, false);
   } else {

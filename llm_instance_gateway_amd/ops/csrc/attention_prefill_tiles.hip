@@ -16,7 +16,10 @@
 // per-position query temperature tau(p) = 1 + c ln(floor((p+1)/e) + 1)
 // multiplies the fp32 scores of row p; the sigmoid output gate is applied in
 // the epilogue.  K and V are staged separately since their rows differ in
-// length.
+// length.  An optional per-head sink starts every row's running max at
+// sink_h and its running sum at one (a key with that unscaled score and no
+// value).  A value row is the first Dv entries of a cache row of v_row
+// entries, so a latent cache can pass its key rows as values.
 
 #include "elem_types.h"
 
@@ -33,12 +36,13 @@ __global__ __launch_bounds__(256) void paged_attention_prefill_tiles_kernel(
     const uint16_t* __restrict__ k_cache,  // [B, Hkv, BS, D]
     const uint16_t* __restrict__ v_cache,  // [B, Hkv, BS, Dv]
     const uint16_t* __restrict__ gate, long gate_stride,  // nullable
+    const float* __restrict__ sink,                       // nullable, [Hq]
     const int* __restrict__ tile_seq, const int* __restrict__ tile_qstart,
     const int* __restrict__ query_start_locs,  // [S+1]
     const int* __restrict__ context_lens,      // [S] after this step's tokens
     const int* __restrict__ block_tables, float scale, float temp_coef,
     float temp_every, int temp_every_int, int num_q_heads, int num_kv_heads,
-    int D, int Dv, int block_size, int max_blocks) {
+    int D, int Dv, int v_row, int block_size, int max_blocks) {
   constexpr int DB = DVP / 16;
   constexpr int KB = DKP / 32;
 
@@ -98,8 +102,8 @@ __global__ __launch_bounds__(256) void paged_attention_prefill_tiles_kernel(
     }
   }
 
-  float m = -INFINITY;
-  float l = 0.0f;
+  float m = sink ? sink[h] : -INFINITY;
+  float l = sink ? 1.0f : 0.0f;
   f32x4_t acc_o[DB];
 #pragma unroll
   for (int db = 0; db < DB; ++db) acc_o[db] = f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -132,7 +136,7 @@ __global__ __launch_bounds__(256) void paged_attention_prefill_tiles_kernel(
       if (t < ctx && d0 < Dv) {
         const size_t base =
             (((size_t)bt[t / block_size] * num_kv_heads + kvh) * block_size +
-             (t % block_size)) * Dv + d0;
+             (t % block_size)) * v_row + d0;
         vval = *reinterpret_cast<const u16x8*>(v_cache + base);
       } else {
 #pragma unroll
@@ -256,13 +260,14 @@ __global__ __launch_bounds__(256) void paged_attention_prefill_tiles_kernel(
 // uses the any-shape kernel).
 extern "C" int lig_paged_attention_prefill_tiles(
     void* out, const void* q, long q_stride, const void* k_cache,
-    const void* v_cache, const void* gate, long gate_stride,
+    const void* v_cache, const void* gate, long gate_stride, const float* sink,
     const int* tile_seq, const int* tile_qstart, const int* query_start_locs,
     const int* context_lens, const int* block_tables, float scale,
     float temp_coef, float temp_every, int temp_every_int, int ntiles,
-    int num_q_heads, int num_kv_heads, int D, int Dv, int block_size,
+    int num_q_heads, int num_kv_heads, int D, int Dv, int v_row, int block_size,
     int max_blocks, hipStream_t stream) {
   if (D % 8 != 0 || Dv % 8 != 0 || D > 128 || Dv > 128 || D <= 0 || Dv <= 0 ||
+      v_row % 8 != 0 || v_row < Dv ||
       q_stride % 8 != 0 || !aligned16(q) || !aligned16(k_cache) ||
       !aligned16(v_cache) || num_q_heads % num_kv_heads != 0)
     return 1;
@@ -274,9 +279,10 @@ extern "C" int lig_paged_attention_prefill_tiles(
                      block, 0, stream, (uint16_t*)out, (const uint16_t*)q,    \
                      q_stride, (const uint16_t*)k_cache,                      \
                      (const uint16_t*)v_cache, (const uint16_t*)gate,         \
-                     gate_stride, tile_seq, tile_qstart, query_start_locs,    \
+                     gate_stride, sink, tile_seq, tile_qstart,                \
+                     query_start_locs,                                        \
                      context_lens, block_tables, scale, temp_coef, temp_every, \
-                     temp_every_int, num_q_heads, num_kv_heads, D, Dv,        \
+                     temp_every_int, num_q_heads, num_kv_heads, D, Dv, v_row, \
                      block_size, max_blocks)
   const int dkp = D <= 32 ? 32 : (D <= 64 ? 64 : 128);
   const int dvp = Dv <= 32 ? 32 : (Dv <= 64 ? 64 : 128);

@@ -1,0 +1,179 @@
+// Offset-weight RMS norms over an fp32 residual with a token shift, and the
+// residual add that goes with a parallel (mixer + feed-forward) layer, gfx950.
+//
+//   n      = x / sqrt(mean(x^2) + eps)              (one statistic per row)
+//   h      = n * (1 + w_mix)                        mixer branch
+//   h_mix  = h + (h_prev - h) * mu                  token shift
+//   h_ff   = n * (1 + w_ff)                         feed-forward branch
+//
+// h_prev is the same quantity of the previous token of the sequence: the row
+// before inside a step's segment (recomputed here from that row, so nothing
+// is exchanged between workgroups), the sequence's state row at a segment's
+// first token (zeros when the sequence starts there).  The workgroup of a
+// segment's FIRST row also refreshes the state with the segment's LAST
+// unblended h after it has read the old one: reader and writer of a state
+// element are the same thread, so a segment of any length needs no second
+// launch.  All arithmetic is fp32; T is the storage type of the weights and
+// of the outputs.
+
+#include "elem_types.h"
+
+#define SN_THREADS 256
+
+template <typename T>
+__global__ __launch_bounds__(SN_THREADS) void offset_norm_shift_kernel(
+    T* __restrict__ h_mix, T* __restrict__ h_ff,  // [R, H]; h_ff nullable
+    const float* __restrict__ x,                  // [R, H]
+    const T* __restrict__ w_mix, const T* __restrict__ w_ff,
+    const T* __restrict__ mu,                     // nullable: no shift
+    float* __restrict__ state,                    // [slots, H]
+    const int* __restrict__ tok_seq, const int* __restrict__ seg_start,
+    const int* __restrict__ seg_len, const int* __restrict__ seg_slot,
+    const int* __restrict__ seg_fresh, float eps, int H) {
+  __shared__ float red[3][17];
+  const int r = blockIdx.x, tid = threadIdx.x;
+  const int s = tok_seq[r];
+  T* om = h_mix + (size_t)r * H;
+  T* of = h_ff ? h_ff + (size_t)r * H : nullptr;
+  if (s < 0) {  // padding row
+    for (int d = tid; d < H; d += SN_THREADS) {
+      st(om + d, 0.f);
+      if (of) st(of + d, 0.f);
+    }
+    return;
+  }
+  const int s0 = seg_start[s], cnt = seg_len[s];
+  const bool first = r == s0;
+  const int r_last = s0 + cnt - 1;
+  const bool shift = mu != nullptr;
+  const bool need_prev = shift && !first;
+  const bool need_last = shift && first && r_last != r;
+  const float* xr = x + (size_t)r * H;
+  const float* xp = x + (size_t)(need_prev ? r - 1 : r) * H;
+  const float* xl = x + (size_t)(need_last ? r_last : r) * H;
+
+  float a = 0.f, b = 0.f, c = 0.f;
+  for (int d = tid; d < H; d += SN_THREADS) {
+    const float v = xr[d];
+    a += v * v;
+    if (need_prev) {
+      const float u = xp[d];
+      b += u * u;
+    }
+    if (need_last) {
+      const float u = xl[d];
+      c += u * u;
+    }
+  }
+  a = block_reduce_sum(a, red[0]);
+  if (need_prev) b = block_reduce_sum(b, red[1]);  // uniform per workgroup
+  if (need_last) c = block_reduce_sum(c, red[2]);
+  const float inv = 1.0f / sqrtf(a / (float)H + eps);
+  const float inv_p = need_prev ? 1.0f / sqrtf(b / (float)H + eps) : 0.f;
+  const float inv_l = need_last ? 1.0f / sqrtf(c / (float)H + eps) : 0.f;
+  float* st_row = shift ? state + (size_t)seg_slot[s] * H : nullptr;
+  const bool fresh = seg_fresh[s] != 0;
+
+  for (int d = tid; d < H; d += SN_THREADS) {
+    const float n = xr[d] * inv;
+    const float g = 1.0f + ld(w_mix + d);
+    const float h = n * g;
+    float o = h;
+    if (shift) {
+      float prev;
+      if (first) {
+        prev = fresh ? 0.f : st_row[d];
+        st_row[d] = need_last ? xl[d] * inv_l * g : h;
+      } else {
+        prev = xp[d] * inv_p * g;
+      }
+      o = h + (prev - h) * ld(mu + d);
+    }
+    st(om + d, o);
+    if (of) st(of + d, n * (1.0f + ld(w_ff + d)));
+  }
+}
+
+// out = x / sqrt(mean(x^2) + eps) * (1 + w), fp32 rows -> storage type
+template <typename T>
+__global__ __launch_bounds__(SN_THREADS) void offset_rms_norm_kernel(
+    T* __restrict__ out, const float* __restrict__ x, const T* __restrict__ w,
+    float eps, int H) {
+  __shared__ float red[17];
+  const int r = blockIdx.x, tid = threadIdx.x;
+  const float* xr = x + (size_t)r * H;
+  float a = 0.f;
+  for (int d = tid; d < H; d += SN_THREADS) a += xr[d] * xr[d];
+  a = block_reduce_sum(a, red);
+  const float inv = 1.0f / sqrtf(a / (float)H + eps);
+  for (int d = tid; d < H; d += SN_THREADS)
+    st(out + (size_t)r * H + d, xr[d] * inv * (1.0f + ld(w + d)));
+}
+
+// x += a (+ b): the fp32 residual takes both branch outputs in one pass
+template <typename T, int N>
+__global__ void residual_add_kernel(float* __restrict__ x, const T* __restrict__ a,
+                                    const T* __restrict__ b, long n) {
+  for (long i = (blockIdx.x * (long)blockDim.x + threadIdx.x) * N; i < n;
+       i += gridDim.x * (long)blockDim.x * N) {
+    float xv[N], av[N], bv[N];
+    ldn<N>(x + i, xv);
+    ldn<N>(a + i, av);
+    if (b) ldn<N>(b + i, bv);
+#pragma unroll
+    for (int k = 0; k < N; ++k) xv[k] += b ? av[k] + bv[k] : av[k];
+    stn<N>(x + i, xv);
+  }
+}
+
+extern "C" {
+
+void lig_offset_norm_shift(void* h_mix, void* h_ff, const float* x,
+                           const void* w_mix, const void* w_ff, const void* mu,
+                           float* state, const int* tok_seq, const int* seg_start,
+                           const int* seg_len, const int* seg_slot,
+                           const int* seg_fresh, float eps, int R, int H,
+                           int is_f32, hipStream_t s) {
+  if (R <= 0) return;
+  if (is_f32)
+    hipLaunchKernelGGL(offset_norm_shift_kernel<float>, dim3(R), dim3(SN_THREADS), 0, s,
+                       (float*)h_mix, (float*)h_ff, x, (const float*)w_mix,
+                       (const float*)w_ff, (const float*)mu, state, tok_seq,
+                       seg_start, seg_len, seg_slot, seg_fresh, eps, H);
+  else
+    hipLaunchKernelGGL(offset_norm_shift_kernel<bf16s>, dim3(R), dim3(SN_THREADS), 0, s,
+                       (bf16s*)h_mix, (bf16s*)h_ff, x, (const bf16s*)w_mix,
+                       (const bf16s*)w_ff, (const bf16s*)mu, state, tok_seq,
+                       seg_start, seg_len, seg_slot, seg_fresh, eps, H);
+}
+
+void lig_offset_rms_norm(void* out, const float* x, const void* w, float eps,
+                         int R, int H, int is_f32, hipStream_t s) {
+  if (R <= 0) return;
+  if (is_f32)
+    hipLaunchKernelGGL(offset_rms_norm_kernel<float>, dim3(R), dim3(SN_THREADS), 0, s,
+                       (float*)out, x, (const float*)w, eps, H);
+  else
+    hipLaunchKernelGGL(offset_rms_norm_kernel<bf16s>, dim3(R), dim3(SN_THREADS), 0, s,
+                       (bf16s*)out, x, (const bf16s*)w, eps, H);
+}
+
+void lig_residual_add(float* x, const void* a, const void* b, long n, int is_f32,
+                      hipStream_t s) {
+  if (n <= 0) return;
+  const bool v4 = n % 4 == 0 && aligned16(x) && aligned16(a) && (!b || aligned16(b));
+  const long items = v4 ? n / 4 : n;
+  long g = (items + 255) / 256;
+  const int grid = (int)(g > 65535 ? 65535 : g);
+#define LIG_RA(T, N)                                                            \
+  hipLaunchKernelGGL((residual_add_kernel<T, N>), dim3(grid), dim3(256), 0, s,  \
+                     x, (const T*)a, (const T*)b, n)
+  if (is_f32) {
+    if (v4) LIG_RA(float, 4); else LIG_RA(float, 1);
+  } else {
+    if (v4) LIG_RA(bf16s, 4); else LIG_RA(bf16s, 1);
+  }
+#undef LIG_RA
+}
+
+}  // extern "C"

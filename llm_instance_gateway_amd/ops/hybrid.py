@@ -30,7 +30,7 @@ CSRC = Path(__file__).resolve().parent / "csrc"
 # extension.
 SOURCES = [
     "group_norm.hip", "xielu.hip", "mingru.hip", "attention_general.hip",
-    "attention_prefill_tiles.hip",
+    "attention_prefill_tiles.hip", "shift_norm.hip", "latent_attention.hip", "ff_act.hip",
 ]
 SO_PATH = PKG / "_hybrid.so"
 
@@ -78,8 +78,16 @@ def _declare(lib: ctypes.CDLL) -> None:
         "lig_sigmoid_gate_mul": [p, p, l, i, i, i, p],
         "lig_mingru_scan": [p, p, p, p, l, p, p, p, p, p, p, i, i, i, i, p],
         "lig_paged_attention_general": [
-            p, p, l, p, p, p, i, p, p, p, l, f, f, f, i, i, i, i, i, i, i, i, p,
+            p, p, l, p, p, p, i, p, p, p, l, p, f, f, f, i, i, i, i, i, i, i, i, i, p,
         ],
+        "lig_offset_norm_shift": [p, p, p, p, p, p, p, p, p, p, p, p, f, i, i, i, p],
+        "lig_offset_rms_norm": [p, p, p, f, i, i, i, p],
+        "lig_residual_add": [p, p, p, l, i, p],
+        "lig_latent_kv_prep": [p, p, l, p, p, p, i, p, p, p, f, i, i, i, i, i, p],
+        "lig_rotate_pack_queries": [p, p, p, i, p, i, i, i, i, i, i, p],
+        "lig_scale_gather_rows": [p, p, p, p, l, i, i, p],
+        "lig_relu_squared": [p, p, l, i, p],
+        "lig_silu_mul": [p, p, l, i, i, p],
         "lig_kv_scatter": [p, p, l, p, p, p, i, i, i, i, i, i, p],
         "lig_temperature_scale_rows": [p, p, l, p, f, f, i, i, i, i, p],
     }
@@ -88,7 +96,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         fn.argtypes = args
         fn.restype = None
     pt = lib.lig_paged_attention_prefill_tiles
-    pt.argtypes = [p, p, l, p, p, p, l, p, p, p, p, p, f, f, f, i, i, i, i, i, i, i, i, p]
+    pt.argtypes = [p, p, l, p, p, p, l, p, p, p, p, p, p, f, f, f, i, i, i, i, i, i, i, i, i, p]
     pt.restype = ctypes.c_int
 
 

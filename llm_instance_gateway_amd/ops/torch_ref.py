@@ -291,9 +291,13 @@ def query_temperature(positions: torch.Tensor, coef: float, every: float) -> tor
 def paged_attention_general(
     q, k_cache, v_cache, block_tables, tok_seq, positions, scale: float,
     num_heads: int, gate=None, temp_coef: float = 0.0, temp_every: float = 1.0,
+    sink=None,
 ):
     """q [R, H*D] (may be a strided view); token r belongs to sequence row
-    tok_seq[r] of block_tables (-1: padding row) and sees keys 0..positions[r]."""
+    tok_seq[r] of block_tables (-1: padding row) and sees keys 0..positions[r].
+    `sink` [H] fp32 adds exp(sink_h) to head h's softmax denominator (a key
+    with that unscaled score and no value).  v_cache may be a view into
+    k_cache's rows."""
     R = q.shape[0]
     nb, G, bs, D = k_cache.shape
     Dv = v_cache.shape[-1]
@@ -325,7 +329,12 @@ def paged_attention_general(
             keyp = torch.arange(L, device=q.device)[None, :]
             mask = keyp > positions[r:e, None]
             sc.masked_fill_(mask[None], float("-inf"))
-            o = torch.bmm(torch.softmax(sc, dim=-1), vf).permute(1, 0, 2).reshape(e - r, H * Dv)
+            if sink is not None:
+                sk = sink.float().view(H, 1, 1).expand(H, e - r, 1)
+                pr = torch.softmax(torch.cat([sc, sk], dim=-1), dim=-1)[..., :-1]
+            else:
+                pr = torch.softmax(sc, dim=-1)
+            o = torch.bmm(pr, vf).permute(1, 0, 2).reshape(e - r, H * Dv)
             if gate is not None:
                 o = o * torch.sigmoid(gate[r:e].float())
             out[r:e] = o.to(out.dtype)
@@ -338,3 +347,115 @@ def temperature_scale_rows(q, positions, coef: float, every: float):
         return q.contiguous().clone()
     tau = query_temperature(positions, coef, every)
     return (q.float() * tau[:, None]).to(q.dtype)
+
+
+# -- token shift, latent attention, sink softmax, routed feed-forward ----------
+
+def _rms_scale(x: torch.Tensor, eps: float) -> torch.Tensor:
+    xf = x.float()
+    return xf * torch.rsqrt(xf.pow(2).mean(dim=-1, keepdim=True) + eps)
+
+
+def residual_add(x, a, b=None) -> torch.Tensor:
+    """x += a (+ b), x fp32 in place."""
+    x.add_(a.float())
+    if b is not None:
+        x.add_(b.float())
+    return x
+
+
+def offset_rms_norm(x, w, eps: float, out_dtype) -> torch.Tensor:
+    """RMS norm whose stored weight is an offset from one."""
+    return (_rms_scale(x, eps) * (1.0 + w.float())).to(out_dtype)
+
+
+def offset_norm_shift(
+    x, w_mix, w_ff, mu, state, tok_seq, seg_start, seg_len, seg_slot, seg_fresh,
+    eps: float, out_dtype,
+):
+    """Two offset-weight RMS norms of the same fp32 rows.  The first one's
+    result h is blended with the previous token's, h + (h_prev - h) * mu:
+    inside a segment h_prev is the row before, at a segment's first row it is
+    the sequence's state (zeros when the sequence starts here); the state
+    then takes the segment's last unblended h.  Rows outside every segment
+    come out zero.  Returns (mixer input, feed-forward input or None)."""
+    n = _rms_scale(x, eps)
+    h = n * (1.0 + w_mix.float())
+    prev = torch.zeros_like(h)
+    live = torch.zeros(h.shape[0], 1, dtype=torch.float32, device=h.device)
+    for s0, cnt, slot, fresh in zip(
+        seg_start.tolist(), seg_len.tolist(), seg_slot.tolist(), seg_fresh.tolist()
+    ):
+        if cnt <= 0:
+            continue
+        if not fresh:
+            prev[s0] = state[slot]
+        prev[s0 + 1 : s0 + cnt] = h[s0 : s0 + cnt - 1]
+        state[slot] = h[s0 + cnt - 1]
+        live[s0 : s0 + cnt] = 1.0
+    hm = (h + (prev - h) * mu.float()) * live
+    hf = None if w_ff is None else (n * (1.0 + w_ff.float()) * live).to(out_dtype)
+    return hm.to(out_dtype), hf
+
+
+def rotary_inv_freq(base: float, dims: int, device=None) -> torch.Tensor:
+    """f_i = base^(-2i/dims), i < dims/2, evaluated in float64, stored fp32."""
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    return torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / dims).float().to(device)
+
+
+def _rotate_pairs(v: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor) -> torch.Tensor:
+    """Interleaved rotation of the first 2*len(inv_freq) entries of the last
+    axis: pair (2i, 2i+1) turns by positions * inv_freq[i] (fp32 angles)."""
+    n = inv_freq.shape[0]
+    out = v.float().clone()
+    ang = positions.float()[:, None] * inv_freq[None, :]
+    c, s = torch.cos(ang), torch.sin(ang)
+    while c.dim() < v.dim():
+        c, s = c.unsqueeze(1), s.unsqueeze(1)
+    a, b = out[..., 0 : 2 * n : 2].clone(), out[..., 1 : 2 * n : 2].clone()
+    out[..., 0 : 2 * n : 2] = a * c - b * s
+    out[..., 1 : 2 * n : 2] = b * c + a * s
+    return out
+
+
+def latent_kv_prep(
+    proj, q_rank: int, kv_rank: int, rot_dim: int, w_q, w_kv, eps: float,
+    inv_freq, positions, slot_mapping, cache,
+):
+    """proj [R, >= q_rank + kv_rank + rot_dim] holds, per row, the query
+    latent, the key/value latent and the shared rotated key part.  Returns
+    the RMS-normed query latent [R, q_rank]; writes the normed key/value
+    latent followed by the rotated key part into cache row slot_mapping[r]
+    (cache [blocks, 1, block_size, kv_rank + rot_dim])."""
+    a, b = q_rank, q_rank + kv_rank
+    cq = (_rms_scale(proj[:, :a], eps) * w_q.float()).to(proj.dtype)
+    c = _rms_scale(proj[:, a:b], eps) * w_kv.float()
+    kr = _rotate_pairs(proj[:, b : b + rot_dim], positions, inv_freq)
+    row = torch.cat([c, kr], dim=-1).to(cache.dtype)
+    ok = slot_mapping >= 0
+    flat = cache.view(-1, kv_rank + rot_dim)
+    flat[slot_mapping[ok]] = row[ok]
+    return cq
+
+
+def rotate_pack_queries(q, heads: int, dim: int, rot_dim: int, inv_freq, positions, out, lead: int):
+    """out[r, h, lead:lead+rot_dim] = rotated q[r, h, dim:dim+rot_dim]; q is
+    [R, heads*(dim+rot_dim)], out [R, heads, lead+rot_dim]."""
+    R = q.shape[0]
+    qr = q.view(R, heads, dim + rot_dim)[:, :, dim:]
+    out[:, :, lead:] = _rotate_pairs(qr, positions, inv_freq).to(out.dtype)
+    return out
+
+
+def relu_squared(x: torch.Tensor) -> torch.Tensor:
+    z = torch.relu(x.float())
+    return (z * z).to(x.dtype)
+
+
+def scale_gather_rows(x, idx, w) -> torch.Tensor:
+    """out[i] = w[i] * x[idx[i]] (fp32 product, rounded to x's dtype); rows
+    with idx < 0 come out zero."""
+    ok = idx >= 0
+    rows = x.float()[idx.clamp(min=0)] * (w.float() * ok)[:, None]
+    return rows.to(x.dtype)
