@@ -138,6 +138,7 @@ class DecodeGraphRunner:
                 seg_len=self.seg_len[:B],
                 seg_slot=self.seg_slot[:B],
                 seg_fresh=self.seg_fresh[:B],
+                seg_ctx=self.context_lens[:B],
                 max_seg_len=1,
             )
         return BatchMeta(

@@ -75,6 +75,7 @@ class BatchMeta:
     seg_len: Optional[torch.Tensor] = None    # [S] int32 tokens it brings this step
     seg_slot: Optional[torch.Tensor] = None   # [S] int32 recurrent-state slot
     seg_fresh: Optional[torch.Tensor] = None  # [S] int32 1 = starts at position 0
+    seg_ctx: Optional[torch.Tensor] = None    # [S] int32 tokens of the sequence after this step
     max_seg_len: int = 0                      # host-side max of seg_len
 
     @property

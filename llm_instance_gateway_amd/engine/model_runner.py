@@ -372,7 +372,9 @@ class ModelRunner:
             s_len: List[int] = []
             s_slot: List[int] = []
             s_fresh: List[int] = []
+            s_ctx: List[int] = []
             for si, ss in enumerate(ordered):
+                s_ctx.append(ss.seq.num_computed_tokens + ss.num_tokens)
                 s_start.append(len(tok_seq))
                 s_len.append(ss.num_tokens)
                 s_slot.append(max(ss.seq.state_slot, 0))
@@ -387,6 +389,7 @@ class ModelRunner:
             meta.tok_seq = i32(tok_seq)
             meta.seg_start, meta.seg_len = i32(s_start), i32(s_len)
             meta.seg_slot, meta.seg_fresh = i32(s_slot), i32(s_fresh)
+            meta.seg_ctx = i32(s_ctx)
             meta.max_seg_len = max(s_len) if s_len else 0
 
         ids_t = torch.tensor(input_ids, dtype=torch.int64).to(dev, non_blocking=True)

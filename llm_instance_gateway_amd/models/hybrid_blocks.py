@@ -288,8 +288,9 @@ class LatentAttention(nn.Module):
                 self.sink.copy_(get(prefix + "sink").float())
             self.w_o.copy_(get(prefix + "o"))
 
-    def tiled_prefill(self, dtype, on_gpu: bool) -> bool:
-        return ops.tiled_prefill_supported(dtype, self.row, self.kv_rank, on_gpu)
+    def mfma_rows(self, dtype, on_gpu: bool) -> bool:
+        return ops.latent_rows_supported(dtype, self.row, self.kv_rank, on_gpu)
+
 
     def forward(self, h, positions, cache, meta):
         lat_cache = cache[0]
@@ -311,23 +312,17 @@ class LatentAttention(nn.Module):
         qa = qa.view(rows, H * self.row)
         v_view = lat_cache[..., :Rk]
         np_ = meta.num_prefill_tokens
-        if (
-            np_ > 0
-            and meta.prefill_tile_seq is not None
-            and self.tiled_prefill(q.dtype, q.is_cuda)
-        ):
-            o = torch.empty(rows, H * Rk, dtype=q.dtype, device=q.device)
-            ops.paged_attention_prefill_tiles(
-                qa[:np_], lat_cache, v_view, meta.prefill_block_tables,
-                meta.prefill_query_start_locs, meta.prefill_context_lens,
-                meta.prefill_tile_seq, meta.prefill_tile_qstart, self.scale, H,
-                sink=self.sink, out=o[:np_],
+        if self.mfma_rows(q.dtype, q.is_cuda) and meta.seg_ctx is not None:
+            # every row of the step in one launch: (token, head) row tiles
+            # that share each key tile across the heads
+            covered = np_ + meta.num_decode_tokens
+            o = (torch.zeros if covered < rows else torch.empty)(
+                rows, H * Rk, dtype=q.dtype, device=q.device
             )
-            if rows > np_:
-                ops.paged_attention_general(
-                    qa[np_:], lat_cache, v_view, meta.seq_block_tables, meta.tok_seq[np_:],
-                    positions[np_:], self.scale, H, sink=self.sink, out=o[np_:],
-                )
+            ops.latent_attention_rows(
+                qa, lat_cache, Rk, meta.seq_block_tables, meta.seg_start, meta.seg_len,
+                meta.seg_ctx, meta.max_seg_len, self.scale, H, sink=self.sink, out=o,
+            )
         else:
             o = ops.paged_attention_general(
                 qa, lat_cache, v_view, meta.seq_block_tables, meta.tok_seq, positions,

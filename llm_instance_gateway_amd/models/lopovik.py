@@ -149,8 +149,8 @@ class LopovikForCausalLM(nn.Module):
             a, b, times = cfg.layer_loop
             self.pass_starts = {a + k * (b - a) for k in range(times)}
             self.loop_in = _param((H, 2 * H), device, dtype, 1.0 / (2 * H) ** 0.5)
-        on_gpu = self.device_.type == "cuda"
-        self.needs_prefill_tiles = any(l.mixer.tiled_prefill(dtype, on_gpu) for l in self.layers)
+        # attention addresses the batch per segment: no per-head query tiles
+        self.needs_prefill_tiles = False
         # test/debug hook: when a list, forward() appends the fp32 residual
         # stream after every layer run
         self.capture_residuals: Optional[list] = None

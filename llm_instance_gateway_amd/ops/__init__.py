@@ -619,6 +619,57 @@ def paged_attention_prefill_tiles(
 
 # -- token shift, latent attention, routed feed-forward -------------------------
 
+def latent_rows_supported(q_dtype, row: int, v_dim: int, is_cuda: bool) -> bool:
+    """The MFMA multi-query kernel over a latent cache: bf16, cache rows of
+    up to 576 entries whose leading v_dim (up to 512) are the values, both
+    multiples of 8."""
+    return (
+        is_cuda
+        and q_dtype == torch.bfloat16
+        and row % 8 == 0
+        and v_dim % 8 == 0
+        and 0 < v_dim <= min(row, 512)
+        and row <= 576
+        and os.environ.get("LIG_FORCE_TORCH_OPS") != "1"
+        and os.environ.get("LIG_GENERAL_ATTENTION") != "1"
+    )
+
+
+def latent_attention_rows(
+    q, cache, v_dim: int, block_tables, seg_start, seg_len, seg_ctx, max_seg_len: int,
+    scale: float, num_heads: int, sink: Optional[torch.Tensor] = None,
+    out: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """Causal multi-query attention of every segment of the step (prompt
+    portions and single tokens alike) over the paged latent cache
+    [blocks, 1, block_size, row]: keys are whole rows, values their leading
+    v_dim entries, all heads of a token share them.  q [R, heads*row]
+    contiguous; segment s covers rows seg_start[s] .. +seg_len[s] of the flat
+    batch, belongs to row s of block_tables and holds seg_ctx[s] tokens after
+    this step.  Rows of no segment are left untouched.  GPU, bf16."""
+    nb, G, bs, row = cache.shape
+    R = q.shape[0]
+    assert G == 1 and q.is_cuda and q.dtype == torch.bfloat16 and cache.dtype == q.dtype
+    assert q.is_contiguous() and q.shape[1] == num_heads * row and cache.is_contiguous()
+    for t in (block_tables, seg_start, seg_len, seg_ctx):
+        assert t.dtype == torch.int32 and t.is_contiguous()
+    S = seg_start.shape[0]
+    assert block_tables.shape[0] >= S and seg_len.shape[0] == S and seg_ctx.shape[0] == S
+    if sink is not None:
+        assert sink.dtype == torch.float32 and sink.shape == (num_heads,) and sink.is_contiguous()
+    if out is None:
+        out = torch.empty(R, num_heads * v_dim, dtype=q.dtype, device=q.device)
+    assert out.shape == (R, num_heads * v_dim) and out.is_contiguous() and out.dtype == q.dtype
+    rc = _hl().lig_latent_attention_rows(
+        _ptr(out), _ptr(q), _ptr(cache), _ptr(sink), _ptr(seg_start), _ptr(seg_len),
+        _ptr(seg_ctx), _ptr(block_tables), block_tables.shape[1], float(scale), S,
+        int(max_seg_len), num_heads, row, v_dim, bs, _stream(),
+    )
+    if rc != 0:
+        raise RuntimeError("latent_attention_rows: shape or alignment not served")
+    return out
+
+
 def residual_add(x: torch.Tensor, a: torch.Tensor, b: Optional[torch.Tensor] = None) -> torch.Tensor:
     """x += a (+ b) in place; x is the fp32 residual, a and b branch outputs."""
     assert x.dtype == torch.float32 and a.shape == x.shape and (b is None or b.shape == x.shape)

@@ -1,0 +1,255 @@
+// Multi-query attention over a paged latent cache on MFMA tiles, bf16, gfx950:
+// every query head of a token reads the SAME cache rows, keys being the whole
+// row (D entries) and values its leading Dv entries.
+//
+// Because all heads share the keys, the query rows of a tile are (token,
+// head) pairs: row rho = token * H + head inside a sequence's segment of the
+// step, 64 consecutive rho per workgroup (4 waves x 16 rows).  A key/value
+// tile is read from HBM/L2 once per workgroup and serves every head in it,
+// so a decode step (one token, H heads) is one pass over the sequence's cache
+// and a prompt portion moves H times fewer key bytes than a per-head grid.
+// Prompt portions and single tokens go through the same kernel: a segment is
+// (first row, token count, context length after the step), and a row's
+// causal bound is its token's position.
+//
+// Per 32-key tile: each 16-byte chunk of a cache row is loaded once and
+// stored twice in LDS, row-major for S^T = K Q^T and transposed for O += P V
+// (mfma_f32_16x16x32_bf16, zero padding to the template's DKP / DVP).
+// Scores, running max and sum are fp32; an optional per-head sink starts a
+// row's running max at sink_h and its sum at one.
+//
+// Grid = (ceil(max segment rows / 64), segments); workgroups past a
+// segment's last row exit at once.
+
+#include "elem_types.h"
+
+typedef __bf16 lr_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float lr_f32x4 __attribute__((ext_vector_type(4)));
+
+#define LR_KVBLK 32
+#define LR_ROWS 64
+
+template <int DKP, int DVP>
+__global__ __launch_bounds__(256) void latent_attention_rows_kernel(
+    uint16_t* __restrict__ out,          // [R, H * Dv]
+    const uint16_t* __restrict__ q,      // [R, H * D] contiguous
+    const uint16_t* __restrict__ cache,  // [blocks, 1, BS, D]
+    const float* __restrict__ sink,      // nullable, [H]
+    const int* __restrict__ seg_start, const int* __restrict__ seg_len,
+    const int* __restrict__ seg_ctx,     // tokens of the sequence after this step
+    const int* __restrict__ block_tables, int max_blocks, float scale, int H,
+    int D, int Dv, int block_size) {
+  static_assert(DVP <= DKP, "values are a prefix of the key row");
+  constexpr int DB = DVP / 16;
+  constexpr int KB = DKP / 32;
+
+  struct Shared {
+    uint16_t K[LR_KVBLK][DKP];
+    uint16_t VT[DVP][LR_KVBLK];
+    uint16_t P[4][16][LR_KVBLK];
+  };
+  __shared__ Shared sm;
+
+  const int s = blockIdx.y;
+  const int n = seg_len[s];
+  const long nrows = (long)n * H;
+  const long rho0 = (long)blockIdx.x * LR_ROWS;
+  if (rho0 >= nrows) return;
+  const long lo = seg_start[s];
+  const int ctx = seg_ctx[s];
+  const int* bt = block_tables + (size_t)s * max_blocks;
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6;
+  const int lane = tid & 63;
+  const int li = lane & 15;
+  const int lg = lane >> 4;
+
+  const long rho = rho0 + wave * 16 + li;
+  const bool row_valid = rho < nrows;
+  const int tok = (int)((row_valid ? rho : rho0) / H);
+  const int head = (int)((row_valid ? rho : rho0) - (long)tok * H);
+  const int qpos = ctx - n + tok;
+
+  lr_bf16x8 q_frag[KB];
+  {
+    const uint16_t* qp = q + ((size_t)lo * H + (row_valid ? rho : rho0)) * D;
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb) {
+      const int d0 = kb * 32 + lg * 8;
+      u16x8 raw;
+      if (d0 < D) {
+        raw = *reinterpret_cast<const u16x8*>(qp + d0);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) raw[e] = 0;
+      }
+      q_frag[kb] = *reinterpret_cast<lr_bf16x8*>(&raw);
+    }
+  }
+
+  float m = sink ? sink[head] : -INFINITY;
+  float l = sink ? 1.0f : 0.0f;
+  lr_f32x4 acc_o[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db) acc_o[db] = lr_f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const long last_rho = (rho0 + LR_ROWS < nrows ? rho0 + LR_ROWS : nrows) - 1;
+  const int kv_end = ctx - n + (int)(last_rho / H) + 1;  // keys any row of the tile sees
+
+  for (int kv0 = 0; kv0 < kv_end; kv0 += LR_KVBLK) {
+    // ---- staging: one load per 16-byte chunk, stored row-major and transposed ----
+    for (int c = tid; c < LR_KVBLK * (DKP / 8); c += 256) {
+      const int row = c / (DKP / 8);
+      const int d0 = (c % (DKP / 8)) * 8;
+      const int t = kv0 + row;
+      u16x8 kval;
+      if (t < kv_end && d0 < D) {
+        const size_t base =
+            ((size_t)bt[t / block_size] * block_size + (t % block_size)) * D + d0;
+        kval = *reinterpret_cast<const u16x8*>(cache + base);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) kval[e] = 0;
+      }
+      *reinterpret_cast<u16x8*>(&sm.K[row][d0]) = kval;
+      if (d0 < DVP) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sm.VT[d0 + e][row] = (d0 + e < Dv) ? kval[e] : (uint16_t)0;
+      }
+    }
+    __syncthreads();
+
+    // ---- S^T = K Q^T ----------------------------------------------------------
+    lr_f32x4 acc_s[2];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+      acc_s[kt] = lr_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb) {
+        u16x8 raw =
+            *reinterpret_cast<const u16x8*>(&sm.K[kt * 16 + li][kb * 32 + lg * 8]);
+        lr_bf16x8 a_frag = *reinterpret_cast<lr_bf16x8*>(&raw);
+        acc_s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+            a_frag, q_frag[kb], acc_s[kt], 0, 0, 0);
+      }
+    }
+
+    // ---- mask + online softmax (this lane owns row rho) -------------------------
+    float sc[8];
+    float rowmax = -INFINITY;
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int key = kv0 + kt * 16 + lg * 4 + r;
+        float v = acc_s[kt][r] * scale;
+        if (!row_valid || key > qpos) v = -INFINITY;
+        sc[kt * 4 + r] = v;
+        rowmax = fmaxf(rowmax, v);
+      }
+    }
+    rowmax = stride_reduce_max<16, 4>(rowmax);
+    const float m_new = fmaxf(m, rowmax);
+    float alpha;
+    float psum = 0.0f;
+    float p[8];
+    if (m_new == -INFINITY) {
+      alpha = 1.0f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) p[i] = 0.0f;
+    } else {
+      alpha = (m == -INFINITY) ? 0.0f : __expf(m - m_new);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        p[i] = (sc[i] == -INFINITY) ? 0.0f : __expf(sc[i] - m_new);
+        psum += p[i];
+      }
+      m = m_new;
+    }
+    psum = stride_reduce_sum<16, 4>(psum);
+    l = l * alpha + psum;
+    // acc_o rows follow the MFMA C layout (row = lg*4 + r); the softmax stats
+    // of row x live in lane x (replicated over the lg groups)
+    float alpha_r[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) alpha_r[r] = __shfl(alpha, lg * 4 + r, 64);
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc_o[db][r] *= alpha_r[r];
+    }
+
+    // ---- P: C layout -> A-fragment layout through the wave's LDS slab ---------
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        sm.P[wave][li][kt * 16 + lg * 4 + r] = f32_to_bf16(p[kt * 4 + r]);
+      }
+    }
+    u16x8 praw = *reinterpret_cast<const u16x8*>(&sm.P[wave][li][lg * 8]);
+    lr_bf16x8 p_frag = *reinterpret_cast<lr_bf16x8*>(&praw);
+
+    // ---- O += P V -----------------------------------------------------------------
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      u16x8 vraw =
+          *reinterpret_cast<const u16x8*>(&sm.VT[db * 16 + li][lg * 8]);
+      lr_bf16x8 v_frag = *reinterpret_cast<lr_bf16x8*>(&vraw);
+      acc_o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(p_frag, v_frag,
+                                                          acc_o[db], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue: normalise and store ------------------------------------------------
+  float inv_l[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const float lr = __shfl(l, lg * 4 + r, 64);  // all lanes active here
+    inv_l[r] = lr > 0.f ? 1.0f / lr : 0.0f;
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const long orho = rho0 + wave * 16 + lg * 4 + r;
+    if (orho >= nrows) continue;
+    uint16_t* op = out + ((size_t)lo * H + orho) * Dv;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      const int d = db * 16 + li;
+      if (d < Dv) op[d] = f32_to_bf16(acc_o[db][r] * inv_l[r]);
+    }
+  }
+}
+
+// Returns 0 when launched, 1 when the shape is not served (the caller then
+// uses another kernel).
+extern "C" int lig_latent_attention_rows(
+    void* out, const void* q, const void* cache, const float* sink,
+    const int* seg_start, const int* seg_len, const int* seg_ctx,
+    const int* block_tables, int max_blocks, float scale, int num_segs,
+    int max_seg_len, int H, int D, int Dv, int block_size, hipStream_t stream) {
+  if (D % 8 != 0 || Dv % 8 != 0 || D <= 0 || Dv <= 0 || Dv > D || D > 576 ||
+      Dv > 512 || !aligned16(q) || !aligned16(cache) || H <= 0)
+    return 1;
+  if (num_segs <= 0 || max_seg_len <= 0) return 0;
+  const long tiles = ((long)max_seg_len * H + LR_ROWS - 1) / LR_ROWS;
+  if (tiles > 2147483647L || num_segs > 65535) return 1;
+  dim3 grid((unsigned)tiles, num_segs);
+  dim3 block(256);
+#define LAUNCH_LR(DKP, DVP)                                                    \
+  hipLaunchKernelGGL((latent_attention_rows_kernel<DKP, DVP>), grid, block, 0, \
+                     stream, (uint16_t*)out, (const uint16_t*)q,               \
+                     (const uint16_t*)cache, sink, seg_start, seg_len,         \
+                     seg_ctx, block_tables, max_blocks, scale, H, D, Dv,       \
+                     block_size)
+  if (D <= 64 && Dv <= 64) LAUNCH_LR(64, 64);
+  else if (D <= 128 && Dv <= 64) LAUNCH_LR(128, 64);
+  else if (D <= 128) LAUNCH_LR(128, 128);
+  else if (D <= 192 && Dv <= 128) LAUNCH_LR(192, 128);
+  else if (D <= 320 && Dv <= 256) LAUNCH_LR(320, 256);
+  else LAUNCH_LR(576, 512);
+#undef LAUNCH_LR
+  return 0;
+}

@@ -31,6 +31,7 @@ CSRC = Path(__file__).resolve().parent / "csrc"
 SOURCES = [
     "group_norm.hip", "xielu.hip", "mingru.hip", "attention_general.hip",
     "attention_prefill_tiles.hip", "shift_norm.hip", "latent_attention.hip", "ff_act.hip",
+    "attention_latent_rows.hip",
 ]
 SO_PATH = PKG / "_hybrid.so"
 
@@ -98,6 +99,9 @@ def _declare(lib: ctypes.CDLL) -> None:
     pt = lib.lig_paged_attention_prefill_tiles
     pt.argtypes = [p, p, l, p, p, p, l, p, p, p, p, p, p, f, f, f, i, i, i, i, i, i, i, i, i, p]
     pt.restype = ctypes.c_int
+    lr = lib.lig_latent_attention_rows
+    lr.argtypes = [p, p, p, p, p, p, p, p, i, f, i, i, i, i, i, i, p]
+    lr.restype = ctypes.c_int
 
 
 def lib() -> ctypes.CDLL:

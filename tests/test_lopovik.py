@@ -68,8 +68,7 @@ CFG_L = {
     "layers": [lat(2, 8, 4, 8, 12, 12, dense(16)), lat(2, 8, 4, 8, 12, 12, moe(4, 3, 8))],
     "loop": {"start": 0, "stop": 2, "times": 1},
 }
-# cache rows the MFMA prompt kernel takes (multiples of 8 up to 128) beside
-# one it does not (row of 136)
+# cache rows of three of the MFMA kernel's size classes (80, 128, 136 entries)
 CFG_C = {
     "architecture": "Lopovik", "vocab": 40, "width": 64, "norm": {"eps": 1e-5},
     "layers": [lat(4, 32, 16, 32, 48, 64, dense(96)), lat(2, 64, 32, 64, 40, 96, moe(4, 2, 32)),
@@ -382,14 +381,14 @@ def test_preempted_sequence_recomputes_its_state(model_a, device):
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_cache_rows_of_the_tiled_kernel(model_c, device, dtype):
+def test_cache_rows_of_the_mfma_kernel(model_c, device, dtype):
     if device == "cpu" and dtype == torch.bfloat16:
         pytest.skip("bf16 is the GPU serving precision")
     ta, tb = tokens_for(CFG_C, 150, 41), tokens_for(CFG_C, 70, 42)
     wa, wb = O.forward(CFG_C, model_c[1], ta), O.forward(CFG_C, model_c[1], tb)
     eng = make_engine(model_c[0], device, dtype)
     if device != "cpu" and dtype == torch.bfloat16:
-        assert eng.runner.model.needs_prefill_tiles
+        assert all(l.mixer.mfma_rows(dtype, True) for l in eng.runner.model.layers)
     got_a, got_b = [], []
     # a: 100-token portion (two 64-row tiles, the second partial), then single
     # tokens; b joins with portions beside a's single tokens

@@ -367,3 +367,56 @@ def test_scored_experts(device, dtype, E, top):
         gt, up = x @ W["e0.gate"].double().T, x @ W["e0.up"].double().T
         out_scaled = s * ((gt * torch.sigmoid(gt) * up) @ W["e0.down"].double().T)
         assert (out_scaled - want).abs().max() > 1e-3
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("row,Dv,H,bs", [(80, 64, 6, 16), (576, 512, 16, 16), (136, 128, 3, 8), (40, 24, 70, 16), (320, 256, 5, 32)])
+def test_latent_rows_kernel(row, Dv, H, bs):
+    """MFMA multi-query kernel, (token, head) row tiles: in one launch a
+    fresh prompt, a portion continuing a long context, a two-token portion
+    and two single tokens (one of them a sequence's first); values are the
+    leading entries of the key rows; sink in the denominator; a loud key at a
+    64-key border; head counts that do not divide the 64-row tile."""
+    dev, dtype = "cuda:0", torch.bfloat16
+    assert ops.latent_rows_supported(dtype, row, Dv, True)
+    g = torch.Generator().manual_seed(row + H)
+    scale = 1.0 / math.sqrt(row)
+    lens, news = [70, 333, 50, 129, 1], [70, 97, 2, 1, 1]
+    nblk = sum((L + bs - 1) // bs for L in lens) + 1
+    cache = torch.zeros(nblk, 1, bs, row, dtype=dtype)
+    tables, keys, at = [], [], 1
+    for L in lens:
+        k = torch.randn(L, row, generator=g)
+        if L > 64:
+            k[64] *= 2.0
+        nb = (L + bs - 1) // bs
+        ids = list(range(at, at + nb))[::-1]
+        at += nb
+        for j in range(L):
+            cache[ids[j // bs], 0, j % bs] = k[j].to(dtype)
+        tables.append(ids)
+        keys.append(k.to(dtype).double())
+    mb = max(len(t) for t in tables)
+    bt = torch.zeros(len(lens), mb, dtype=torch.int32)
+    for i, t in enumerate(tables):
+        bt[i, : len(t)] = torch.tensor(t)
+    starts = [0]
+    for n in news:
+        starts.append(starts[-1] + n)
+    R = starts[-1] + 3  # three rows of no segment at the end
+    q = torch.randn(R, H * row, generator=g).to(dtype)
+    sink = torch.randn(H, generator=g) * 2
+    out = torch.full((R, H * Dv), 9.0, dtype=dtype, device=dev)
+    ops.latent_attention_rows(
+        q.to(dev), cache.to(dev), Dv, bt.to(dev), i32(starts[:-1], dev), i32(news, dev), i32(lens, dev),
+        max(news), scale, H, sink=sink.to(dev), out=out,
+    )
+    got = out.cpu()
+    assert float((got[starts[-1]:].float() - 9.0).abs().max()) == 0.0, "rows of no segment are left alone"
+    for s, (L, n) in enumerate(zip(lens, news)):
+        for r in sorted({0, 1 % n, n // 2, n - 1}):
+            p = L - n + r
+            qf = q[starts[s] + r].double().view(1, H, row).expand(p + 1, H, row).clone()
+            k = keys[s][: p + 1, None, :].expand(p + 1, H, row)
+            want = O.sink_softmax_attention(qf, k, k[..., :Dv], scale, sink.double())[-1]
+            close(got[starts[s] + r].view(H, Dv), want, dtype, scale=1.0)
