@@ -107,7 +107,26 @@ def main() -> None:
         "PARTS = engine, kernels or both (benchmarks/bench_hybrid.py)",
     )
     ap.add_argument("--hybrid-sizes", default="s,m")
+    ap.add_argument(
+        "--latent",
+        nargs="?",
+        const="engine,kernels",
+        default="",
+        metavar="PARTS",
+        help="instead of the serving workload: Lopovik (latent attention, "
+        "parallel layers) beside Llama and Mixtral at equal size, and its "
+        "kernels beside their counterparts against the roofline; PARTS = "
+        "engine, kernels or both (benchmarks/bench_latent.py)",
+    )
+    ap.add_argument("--latent-sizes", default="s,m")
     args = ap.parse_args()
+
+    if args.latent:
+        sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "benchmarks"))
+        import bench_latent
+
+        bench_latent.main(["--part", args.latent, "--sizes", args.latent_sizes])
+        return
 
     if args.hybrid:
         sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "benchmarks"))

@@ -15,6 +15,10 @@
 // Per 32-key tile: each 16-byte chunk of a cache row is loaded once and
 // stored twice in LDS, row-major for S^T = K Q^T and transposed for O += P V
 // (mfma_f32_16x16x32_bf16, zero padding to the template's DKP / DVP).
+// Consecutive lanes stage consecutive KEYS of one chunk column, so the
+// transposed 2-byte stores of a wave fall into consecutive LDS words; LDS
+// rows are padded by 16 bytes so that the 16-byte fragment reads of 16
+// different rows spread over all banks.
 // Scores, running max and sum are fp32; an optional per-head sink starts a
 // row's running max at sink_h and its sum at one.
 //
@@ -28,6 +32,7 @@ typedef float lr_f32x4 __attribute__((ext_vector_type(4)));
 
 #define LR_KVBLK 32
 #define LR_ROWS 64
+#define LR_PAD 8
 
 template <int DKP, int DVP>
 __global__ __launch_bounds__(256) void latent_attention_rows_kernel(
@@ -44,9 +49,9 @@ __global__ __launch_bounds__(256) void latent_attention_rows_kernel(
   constexpr int KB = DKP / 32;
 
   struct Shared {
-    uint16_t K[LR_KVBLK][DKP];
-    uint16_t VT[DVP][LR_KVBLK];
-    uint16_t P[4][16][LR_KVBLK];
+    uint16_t K[LR_KVBLK][DKP + LR_PAD];
+    uint16_t VT[DVP][LR_KVBLK + LR_PAD];
+    uint16_t P[4][16][LR_KVBLK + LR_PAD];
   };
   __shared__ Shared sm;
 
@@ -100,8 +105,8 @@ __global__ __launch_bounds__(256) void latent_attention_rows_kernel(
   for (int kv0 = 0; kv0 < kv_end; kv0 += LR_KVBLK) {
     // ---- staging: one load per 16-byte chunk, stored row-major and transposed ----
     for (int c = tid; c < LR_KVBLK * (DKP / 8); c += 256) {
-      const int row = c / (DKP / 8);
-      const int d0 = (c % (DKP / 8)) * 8;
+      const int row = c % LR_KVBLK;
+      const int d0 = (c / LR_KVBLK) * 8;
       const int t = kv0 + row;
       u16x8 kval;
       if (t < kv_end && d0 < D) {

@@ -94,6 +94,123 @@ __global__ __launch_bounds__(SN_THREADS) void offset_norm_shift_kernel(
   }
 }
 
+
+// Vector path: H % 4 == 0 and H <= 4 * SN_THREADS * VPT.  Every thread keeps
+// its float4 chunks of the row (and of the neighbouring row it needs) in
+// registers between the reduction and the scaling, so each operand crosses
+// the memory system once; the three sums share one LDS exchange.
+template <typename T, int VPT>
+__global__ __launch_bounds__(SN_THREADS) void offset_norm_shift_vec_kernel(
+    T* __restrict__ h_mix, T* __restrict__ h_ff, const float* __restrict__ x,
+    const T* __restrict__ w_mix, const T* __restrict__ w_ff, const T* __restrict__ mu,
+    float* __restrict__ state, const int* __restrict__ tok_seq,
+    const int* __restrict__ seg_start, const int* __restrict__ seg_len,
+    const int* __restrict__ seg_slot, const int* __restrict__ seg_fresh, float eps,
+    int H) {
+  __shared__ float red[3][SN_THREADS / WAVE_SIZE];
+  const int r = blockIdx.x, tid = threadIdx.x;
+  const int s = tok_seq[r];
+  const int nvec = H / 4;
+  T* om = h_mix + (size_t)r * H;
+  T* of = h_ff ? h_ff + (size_t)r * H : nullptr;
+  if (s < 0) {  // padding row
+    const float z[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int v = tid; v < nvec; v += SN_THREADS) {
+      stn<4>(om + 4 * v, z);
+      if (of) stn<4>(of + 4 * v, z);
+    }
+    return;
+  }
+  const int s0 = seg_start[s], cnt = seg_len[s];
+  const bool first = r == s0;
+  const int r_last = s0 + cnt - 1;
+  const bool shift = mu != nullptr;
+  const bool need_prev = shift && !first;
+  const bool need_last = shift && first && r_last != r;
+  const bool need_other = need_prev || need_last;  // never both
+  const float* xr = x + (size_t)r * H;
+  const float* xo = x + (size_t)(need_prev ? r - 1 : (need_last ? r_last : r)) * H;
+
+  float a[VPT][4], b[VPT][4];
+  float sa = 0.f, sb = 0.f;
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) {
+    const int v = tid + k * SN_THREADS;
+    if (v < nvec) {
+      ldn<4>(xr + 4 * v, a[k]);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) sa += a[k][e] * a[k][e];
+      if (need_other) {
+        ldn<4>(xo + 4 * v, b[k]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sb += b[k][e] * b[k][e];
+      }
+    }
+  }
+  sa = wave_reduce_sum(sa);
+  sb = wave_reduce_sum(sb);
+  const int wave = tid / WAVE_SIZE, lane = tid % WAVE_SIZE;
+  if (lane == 0) {
+    red[0][wave] = sa;
+    red[1][wave] = sb;
+  }
+  __syncthreads();
+  sa = 0.f;
+  sb = 0.f;
+#pragma unroll
+  for (int w = 0; w < SN_THREADS / WAVE_SIZE; ++w) {
+    sa += red[0][w];
+    sb += red[1][w];
+  }
+  const float inv = 1.0f / sqrtf(sa / (float)H + eps);
+  const float inv_o = need_other ? 1.0f / sqrtf(sb / (float)H + eps) : 0.f;
+  float* st_row = shift ? state + (size_t)seg_slot[s] * H : nullptr;
+  const bool fresh = seg_fresh[s] != 0;
+
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) {
+    const int v = tid + k * SN_THREADS;
+    if (v >= nvec) continue;
+    float g[4], o[4], f[4];
+    ldn<4>(w_mix + 4 * v, g);
+    if (shift) {
+      float m4[4], prev[4];
+      ldn<4>(mu + 4 * v, m4);
+      if (first) {
+        if (fresh) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) prev[e] = 0.f;
+        } else {
+          ldn<4>(st_row + 4 * v, prev);
+        }
+        float keep[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          keep[e] = need_last ? b[k][e] * inv_o * (1.0f + g[e]) : a[k][e] * inv * (1.0f + g[e]);
+        stn<4>(st_row + 4 * v, keep);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) prev[e] = b[k][e] * inv_o * (1.0f + g[e]);
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float h = a[k][e] * inv * (1.0f + g[e]);
+        o[e] = h + (prev[e] - h) * m4[e];
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = a[k][e] * inv * (1.0f + g[e]);
+    }
+    stn<4>(om + 4 * v, o);
+    if (of) {
+      ldn<4>(w_ff + 4 * v, f);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) f[e] = a[k][e] * inv * (1.0f + f[e]);
+      stn<4>(of + 4 * v, f);
+    }
+  }
+}
+
 // out = x / sqrt(mean(x^2) + eps) * (1 + w), fp32 rows -> storage type
 template <typename T>
 __global__ __launch_bounds__(SN_THREADS) void offset_rms_norm_kernel(
@@ -135,6 +252,27 @@ void lig_offset_norm_shift(void* h_mix, void* h_ff, const float* x,
                            const int* seg_fresh, float eps, int R, int H,
                            int is_f32, hipStream_t s) {
   if (R <= 0) return;
+  const bool al = aligned16(h_mix) && aligned16(x) && aligned16(w_mix) && aligned16(state) &&
+                  (!h_ff || (aligned16(h_ff) && aligned16(w_ff))) && (!mu || aligned16(mu));
+  if (H % 4 == 0 && H <= 4 * SN_THREADS * 8 && al) {
+    const int vpt = (H / 4 + SN_THREADS - 1) / SN_THREADS;
+#define LIG_SNV(T, V)                                                            \
+  hipLaunchKernelGGL((offset_norm_shift_vec_kernel<T, V>), dim3(R),              \
+                     dim3(SN_THREADS), 0, s, (T*)h_mix, (T*)h_ff, x,             \
+                     (const T*)w_mix, (const T*)w_ff, (const T*)mu, state,       \
+                     tok_seq, seg_start, seg_len, seg_slot, seg_fresh, eps, H)
+#define LIG_SNV_PICK(T)                                                          \
+  do {                                                                           \
+    if (vpt <= 1) LIG_SNV(T, 1);                                                 \
+    else if (vpt <= 2) LIG_SNV(T, 2);                                            \
+    else if (vpt <= 4) LIG_SNV(T, 4);                                            \
+    else LIG_SNV(T, 8);                                                          \
+  } while (0)
+    if (is_f32) LIG_SNV_PICK(float); else LIG_SNV_PICK(bf16s);
+#undef LIG_SNV_PICK
+#undef LIG_SNV
+    return;
+  }
   if (is_f32)
     hipLaunchKernelGGL(offset_norm_shift_kernel<float>, dim3(R), dim3(SN_THREADS), 0, s,
                        (float*)h_mix, (float*)h_ff, x, (const float*)w_mix,

@@ -26,11 +26,11 @@ def skip_cpu_bf16(device, dtype):
         pytest.skip("bf16 is the GPU serving precision")
 
 
-def close(got, want, dtype, scale=None):
+def close(got, want, dtype, scale=None, tol32=2e-5):
     want = want.to(F64)
     s = scale if scale is not None else max(want.abs().max().item(), 1e-6)
     e = (got.detach().double().cpu() - want).abs().max().item() / s
-    assert e < (2e-5 if dtype == torch.float32 else 2e-2), e
+    assert e < (tol32 if dtype == torch.float32 else 2e-2), e
 
 
 def i32(v, device):
@@ -41,7 +41,7 @@ def i32(v, device):
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H", [20, 257])
+@pytest.mark.parametrize("H", [20, 257, 1028, 2560, 5000])  # scalar and 4-wide paths, 1..8 vectors per thread
 def test_offset_norm_shift_over_portions(device, dtype, H):
     """Two sequences fed in portions of 1, 2 and more tokens through reused
     slots; the blended rows equal the whole-sequence computation."""
@@ -135,13 +135,15 @@ def test_residual_add_and_activations(device, dtype, n):
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("sizes", [(10, 6, 4, 4), (24, 16, 8, 4), (5, 3, 2, 0), (300, 260, 6, 6)])
+@pytest.mark.parametrize("sizes", [(10, 6, 4, 4), (24, 16, 8, 4), (5, 3, 2, 0), (300, 260, 6, 6), (1544, 72, 16, 16)])
 def test_latent_prep_writes_normed_latent_and_rotated_key(device, dtype, sizes):
     skip_cpu_bf16(device, dtype)
     q_rank, kv_rank, rot_dim, rot_dims = sizes
     g = torch.Generator().manual_seed(sum(sizes))
     R, bs, nblk, eps, base = 6, 4, 5, 1e-5, 300.0
-    extra = 7  # columns after the three parts (an output gate in the model)
+    # columns after the three parts (an output gate in the model); rows stay
+    # 16-byte aligned when every size is a multiple of 8 (the wave-per-row path)
+    extra = 8 if all(v % 8 == 0 for v in sizes) else 7
     proj = torch.randn(R, q_rank + kv_rank + rot_dim + extra, generator=g).to(dtype)
     wq = (1 + 0.2 * torch.randn(q_rank, generator=g)).to(dtype)
     wkv = (1 + 0.2 * torch.randn(kv_rank, generator=g)).to(dtype)
@@ -168,16 +170,19 @@ def test_latent_prep_writes_normed_latent_and_rotated_key(device, dtype, sizes):
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_rotate_pack_queries(device, dtype):
+@pytest.mark.parametrize("shape", [(6, 8, 6, 10), (8, 16, 16, 24), (16, 24, 10, 8)])
+def test_rotate_pack_queries(device, dtype, shape):
     skip_cpu_bf16(device, dtype)
     g = torch.Generator().manual_seed(5)
-    R, H, D, Rr, dims, lead, base = 5, 3, 6, 8, 6, 10, 1000.0
+    D, Rr, dims, lead = shape
+    R, H, base = 5, 3, 1000.0
     q = torch.randn(R, H * (D + Rr), generator=g).to(dtype)
     pos = torch.tensor([0, 3, 64, 1500, 7], dtype=torch.int64)
     out = torch.zeros(R, H, lead + Rr, dtype=dtype, device=device)
     ops.rotate_pack_queries(q.to(device), H, D, Rr, ops.rotary_inv_freq(base, dims, device), pos.to(device), out, lead)
     want = O.rotate_interleaved(q.double().view(R, H, D + Rr)[..., D:], pos, base, dims)
-    close(out[..., lead:], want, dtype)
+    # angles are fp32 products: at position 1500 their rounding alone is 1e-4 rad
+    close(out[..., lead:], want, dtype, tol32=2e-4)
     assert float(out[..., :lead].abs().max()) == 0.0
     # the last rot_dim - dims entries pass unchanged
     assert torch.equal(out[..., lead + dims :].cpu(), q.view(R, H, D + Rr)[..., D + dims :])
