@@ -4,7 +4,7 @@ throughput through the engine, and the design's kernels beside their
 counterparts against the roofline.
 
     python bench.py --latent                  # both parts, JSON lines
-    python benchmarks/bench_latent.py --part engine|kernels [--sizes s,m]
+    python benchmarks/bench_latent.py --part engine|kernels|profile [--sizes s,m]
 
 Engine part, per size: a Lopovik stack with squared-ReLU feed-forwards beside
 a Llama stack of the same width, depth, head count and feed-forward
@@ -212,6 +212,12 @@ def main(argv=None) -> None:
         part_kernels(sizes)
     if "engine" in args.part:
         part_engine(sizes)
+    if "profile" in args.part:
+        # one model only (routed variant): the run to put under a profiler
+        for name in sizes:
+            print(json.dumps({"bench": "profile", "size": name,
+                              "lopovik_routed": engine_run(lopovik_config(name, SIZES[name], True), 16, 1024, 64)}),
+                  flush=True)
 
 
 if __name__ == "__main__":

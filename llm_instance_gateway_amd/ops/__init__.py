@@ -635,10 +635,20 @@ def latent_rows_supported(q_dtype, row: int, v_dim: int, is_cuda: bool) -> bool:
     )
 
 
+def latent_rows_nsplit(rows: int, segs: int, heads: int, max_ctx: int) -> int:
+    """Context slices for the latent row kernel: 1 when the step's rows fill
+    the chip by themselves, else enough slices for about two workgroups per
+    CU, each with at least 128 keys of the longest possible context."""
+    blocks = (rows * heads + 63) // 64 + segs
+    if blocks >= _NUM_CUS or max_ctx < 512:
+        return 1
+    return max(1, min(32, (2 * _NUM_CUS + blocks - 1) // blocks, max_ctx // 128))
+
+
 def latent_attention_rows(
     q, cache, v_dim: int, block_tables, seg_start, seg_len, seg_ctx, max_seg_len: int,
     scale: float, num_heads: int, sink: Optional[torch.Tensor] = None,
-    out: Optional[torch.Tensor] = None,
+    out: Optional[torch.Tensor] = None, nsplit: int = 0,
 ) -> torch.Tensor:
     """Causal multi-query attention of every segment of the step (prompt
     portions and single tokens alike) over the paged latent cache
@@ -646,7 +656,10 @@ def latent_attention_rows(
     v_dim entries, all heads of a token share them.  q [R, heads*row]
     contiguous; segment s covers rows seg_start[s] .. +seg_len[s] of the flat
     batch, belongs to row s of block_tables and holds seg_ctx[s] tokens after
-    this step.  Rows of no segment are left untouched.  GPU, bf16."""
+    this step.  Rows of no segment are left untouched.  nsplit > 1 cuts every
+    tile's visible keys into that many slices run by separate workgroups and
+    merged afterwards (0: chosen from the row count and the longest context
+    the block tables can hold).  GPU, bf16."""
     nb, G, bs, row = cache.shape
     R = q.shape[0]
     assert G == 1 and q.is_cuda and q.dtype == torch.bfloat16 and cache.dtype == q.dtype
@@ -660,10 +673,15 @@ def latent_attention_rows(
     if out is None:
         out = torch.empty(R, num_heads * v_dim, dtype=q.dtype, device=q.device)
     assert out.shape == (R, num_heads * v_dim) and out.is_contiguous() and out.dtype == q.dtype
+    if nsplit <= 0:
+        nsplit = latent_rows_nsplit(R, S, num_heads, block_tables.shape[1] * bs)
+    scratch = None
+    if nsplit > 1:
+        scratch = split_scratch(q.device, R * num_heads * nsplit * (v_dim + 2))
     rc = _hl().lig_latent_attention_rows(
         _ptr(out), _ptr(q), _ptr(cache), _ptr(sink), _ptr(seg_start), _ptr(seg_len),
         _ptr(seg_ctx), _ptr(block_tables), block_tables.shape[1], float(scale), S,
-        int(max_seg_len), num_heads, row, v_dim, bs, _stream(),
+        int(max_seg_len), num_heads, row, v_dim, bs, int(nsplit), _ptr(scratch), _stream(),
     )
     if rc != 0:
         raise RuntimeError("latent_attention_rows: shape or alignment not served")

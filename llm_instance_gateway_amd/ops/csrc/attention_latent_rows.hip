@@ -22,8 +22,12 @@
 // Scores, running max and sum are fp32; an optional per-head sink starts a
 // row's running max at sink_h and its sum at one.
 //
-// Grid = (ceil(max segment rows / 64), segments); workgroups past a
-// segment's last row exit at once.
+// Grid = (ceil(max segment rows / 64), segments, splits); workgroups past a
+// segment's last row exit at once.  With splits > 1 (few rows, long
+// contexts) each z-slice walks an equal share of the tile's visible keys and
+// leaves its unnormalised sum with its running max and sum in an fp32
+// scratch; a second kernel merges the slices.  The sink is counted by slice
+// zero only.
 
 #include "elem_types.h"
 
@@ -43,7 +47,8 @@ __global__ __launch_bounds__(256) void latent_attention_rows_kernel(
     const int* __restrict__ seg_start, const int* __restrict__ seg_len,
     const int* __restrict__ seg_ctx,     // tokens of the sequence after this step
     const int* __restrict__ block_tables, int max_blocks, float scale, int H,
-    int D, int Dv, int block_size) {
+    int D, int Dv, int block_size, int nsplit,
+    float* __restrict__ partial) {  // [R * H, nsplit, Dv + 2] when nsplit > 1
   static_assert(DVP <= DKP, "values are a prefix of the key row");
   constexpr int DB = DVP / 16;
   constexpr int KB = DKP / 32;
@@ -72,6 +77,8 @@ __global__ __launch_bounds__(256) void latent_attention_rows_kernel(
 
   const long rho = rho0 + wave * 16 + li;
   const bool row_valid = rho < nrows;
+  // a wave whose 16 rows all lie past the segment only helps staging
+  const bool wave_active = rho0 + wave * 16 < nrows;
   const int tok = (int)((row_valid ? rho : rho0) / H);
   const int head = (int)((row_valid ? rho : rho0) - (long)tok * H);
   const int qpos = ctx - n + tok;
@@ -93,8 +100,10 @@ __global__ __launch_bounds__(256) void latent_attention_rows_kernel(
     }
   }
 
-  float m = sink ? sink[head] : -INFINITY;
-  float l = sink ? 1.0f : 0.0f;
+  const int z = blockIdx.z;
+  const bool with_sink = sink != nullptr && z == 0;
+  float m = with_sink ? sink[head] : -INFINITY;
+  float l = with_sink ? 1.0f : 0.0f;
   lr_f32x4 acc_o[DB];
 #pragma unroll
   for (int db = 0; db < DB; ++db) acc_o[db] = lr_f32x4{0.f, 0.f, 0.f, 0.f};
@@ -102,7 +111,15 @@ __global__ __launch_bounds__(256) void latent_attention_rows_kernel(
   const long last_rho = (rho0 + LR_ROWS < nrows ? rho0 + LR_ROWS : nrows) - 1;
   const int kv_end = ctx - n + (int)(last_rho / H) + 1;  // keys any row of the tile sees
 
-  for (int kv0 = 0; kv0 < kv_end; kv0 += LR_KVBLK) {
+  int kv_lo = 0, kv_hi = kv_end;
+  if (nsplit > 1) {
+    const int nt = (kv_end + LR_KVBLK - 1) / LR_KVBLK;
+    const int per = (nt + nsplit - 1) / nsplit;
+    kv_lo = min(kv_end, z * per * LR_KVBLK);
+    kv_hi = min(kv_end, kv_lo + per * LR_KVBLK);
+  }
+
+  for (int kv0 = kv_lo; kv0 < kv_hi; kv0 += LR_KVBLK) {
     // ---- staging: one load per 16-byte chunk, stored row-major and transposed ----
     for (int c = tid; c < LR_KVBLK * (DKP / 8); c += 256) {
       const int row = c % LR_KVBLK;
@@ -125,6 +142,7 @@ __global__ __launch_bounds__(256) void latent_attention_rows_kernel(
     }
     __syncthreads();
 
+    if (wave_active) {
     // ---- S^T = K Q^T ----------------------------------------------------------
     lr_f32x4 acc_s[2];
 #pragma unroll
@@ -205,7 +223,30 @@ __global__ __launch_bounds__(256) void latent_attention_rows_kernel(
       acc_o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(p_frag, v_frag,
                                                           acc_o[db], 0, 0, 0);
     }
+    }  // wave_active
     __syncthreads();
+  }
+
+  if (nsplit > 1) {
+    // ---- partial result: unnormalised sums, running max and sum -------------------
+    const size_t stride = (size_t)Dv + 2;
+    if (row_valid && lg == 0) {
+      float* pp = partial + (((size_t)lo * H + rho) * nsplit + z) * stride;
+      pp[Dv] = m;
+      pp[Dv + 1] = l;
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const long orho = rho0 + wave * 16 + lg * 4 + r;
+      if (orho >= nrows) continue;
+      float* pp = partial + (((size_t)lo * H + orho) * nsplit + z) * stride;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const int d = db * 16 + li;
+        if (d < Dv) pp[d] = acc_o[db][r];
+      }
+    }
+    return;
   }
 
   // ---- epilogue: normalise and store ------------------------------------------------
@@ -228,27 +269,62 @@ __global__ __launch_bounds__(256) void latent_attention_rows_kernel(
   }
 }
 
+
+// Merge the z-slices of every row: m* = max m_z, out = sum_z e^(m_z - m*) acc_z
+// / sum_z e^(m_z - m*) l_z.  One wave per row, lanes over the value entries.
+__global__ __launch_bounds__(256) void latent_attention_rows_combine_kernel(
+    uint16_t* __restrict__ out, const float* __restrict__ partial,
+    const int* __restrict__ seg_start, const int* __restrict__ seg_len, int H,
+    int Dv, int nsplit) {
+  const int s = blockIdx.y;
+  const long nrows = (long)seg_len[s] * H;
+  const long rho = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (rho >= nrows) return;
+  const int lane = threadIdx.x & 63;
+  const size_t g = (size_t)seg_start[s] * H + rho;
+  const size_t stride = (size_t)Dv + 2;
+  const float* pp = partial + g * nsplit * stride;
+  float mstar = -INFINITY;
+  for (int zz = 0; zz < nsplit; ++zz) mstar = fmaxf(mstar, pp[zz * stride + Dv]);
+  float lsum = 0.f;
+  for (int zz = 0; zz < nsplit; ++zz) {
+    const float mz = pp[zz * stride + Dv];
+    if (mz != -INFINITY) lsum += __expf(mz - mstar) * pp[zz * stride + Dv + 1];
+  }
+  const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
+  for (int d = lane; d < Dv; d += 64) {
+    float a = 0.f;
+    for (int zz = 0; zz < nsplit; ++zz) {
+      const float mz = pp[zz * stride + Dv];
+      if (mz != -INFINITY) a += __expf(mz - mstar) * pp[zz * stride + d];
+    }
+    out[g * Dv + d] = f32_to_bf16(a * inv);
+  }
+}
+
 // Returns 0 when launched, 1 when the shape is not served (the caller then
 // uses another kernel).
 extern "C" int lig_latent_attention_rows(
     void* out, const void* q, const void* cache, const float* sink,
     const int* seg_start, const int* seg_len, const int* seg_ctx,
     const int* block_tables, int max_blocks, float scale, int num_segs,
-    int max_seg_len, int H, int D, int Dv, int block_size, hipStream_t stream) {
+    int max_seg_len, int H, int D, int Dv, int block_size, int nsplit,
+    float* partial, hipStream_t stream) {
   if (D % 8 != 0 || Dv % 8 != 0 || D <= 0 || Dv <= 0 || Dv > D || D > 576 ||
       Dv > 512 || !aligned16(q) || !aligned16(cache) || H <= 0)
     return 1;
   if (num_segs <= 0 || max_seg_len <= 0) return 0;
   const long tiles = ((long)max_seg_len * H + LR_ROWS - 1) / LR_ROWS;
   if (tiles > 2147483647L || num_segs > 65535) return 1;
-  dim3 grid((unsigned)tiles, num_segs);
+  if (nsplit < 1 || nsplit > 64 || (nsplit > 1 && partial == nullptr)) return 1;
+  dim3 grid((unsigned)tiles, num_segs, nsplit);
   dim3 block(256);
 #define LAUNCH_LR(DKP, DVP)                                                    \
   hipLaunchKernelGGL((latent_attention_rows_kernel<DKP, DVP>), grid, block, 0, \
                      stream, (uint16_t*)out, (const uint16_t*)q,               \
                      (const uint16_t*)cache, sink, seg_start, seg_len,         \
                      seg_ctx, block_tables, max_blocks, scale, H, D, Dv,       \
-                     block_size)
+                     block_size, nsplit, partial)
   if (D <= 64 && Dv <= 64) LAUNCH_LR(64, 64);
   else if (D <= 128 && Dv <= 64) LAUNCH_LR(128, 64);
   else if (D <= 128) LAUNCH_LR(128, 128);
@@ -256,5 +332,11 @@ extern "C" int lig_latent_attention_rows(
   else if (D <= 320 && Dv <= 256) LAUNCH_LR(320, 256);
   else LAUNCH_LR(576, 512);
 #undef LAUNCH_LR
+  if (nsplit > 1) {
+    const long rows4 = ((long)max_seg_len * H + 3) / 4;
+    hipLaunchKernelGGL(latent_attention_rows_combine_kernel,
+                       dim3((unsigned)rows4, num_segs), dim3(256), 0, stream,
+                       (uint16_t*)out, partial, seg_start, seg_len, H, Dv, nsplit);
+  }
   return 0;
 }

@@ -100,7 +100,7 @@ def _declare(lib: ctypes.CDLL) -> None:
     pt.argtypes = [p, p, l, p, p, p, l, p, p, p, p, p, p, f, f, f, i, i, i, i, i, i, i, i, i, p]
     pt.restype = ctypes.c_int
     lr = lib.lig_latent_attention_rows
-    lr.argtypes = [p, p, p, p, p, p, p, p, i, f, i, i, i, i, i, i, p]
+    lr.argtypes = [p, p, p, p, p, p, p, p, i, f, i, i, i, i, i, i, i, p, p]
     lr.restype = ctypes.c_int
 
 

@@ -375,13 +375,16 @@ def test_scored_experts(device, dtype, E, top):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("nsplit", [1, 3, 8])
 @pytest.mark.parametrize("row,Dv,H,bs", [(80, 64, 6, 16), (576, 512, 16, 16), (136, 128, 3, 8), (40, 24, 70, 16), (320, 256, 5, 32)])
-def test_latent_rows_kernel(row, Dv, H, bs):
+def test_latent_rows_kernel(row, Dv, H, bs, nsplit):
     """MFMA multi-query kernel, (token, head) row tiles: in one launch a
     fresh prompt, a portion continuing a long context, a two-token portion
     and two single tokens (one of them a sequence's first); values are the
     leading entries of the key rows; sink in the denominator; a loud key at a
-    64-key border; head counts that do not divide the 64-row tile."""
+    64-key border; head counts that do not divide the 64-row tile.  With
+    nsplit > 1 the visible keys of a tile are cut into slices merged by a
+    second kernel (slices of a one-key context are empty but for the first)."""
     dev, dtype = "cuda:0", torch.bfloat16
     assert ops.latent_rows_supported(dtype, row, Dv, True)
     g = torch.Generator().manual_seed(row + H)
@@ -414,7 +417,7 @@ def test_latent_rows_kernel(row, Dv, H, bs):
     out = torch.full((R, H * Dv), 9.0, dtype=dtype, device=dev)
     ops.latent_attention_rows(
         q.to(dev), cache.to(dev), Dv, bt.to(dev), i32(starts[:-1], dev), i32(news, dev), i32(lens, dev),
-        max(news), scale, H, sink=sink.to(dev), out=out,
+        max(news), scale, H, sink=sink.to(dev), out=out, nsplit=nsplit,
     )
     got = out.cpu()
     assert float((got[starts[-1]:].float() - 9.0).abs().max()) == 0.0, "rows of no segment are left alone"
