@@ -677,7 +677,7 @@ def latent_attention_rows(
         nsplit = latent_rows_nsplit(R, S, num_heads, block_tables.shape[1] * bs)
     scratch = None
     if nsplit > 1:
-        scratch = split_scratch(q.device, R * num_heads * nsplit * (v_dim + 2))
+        scratch = split_scratch(q.device, R * num_heads * nsplit * (v_dim + 4))
     rc = _hl().lig_latent_attention_rows(
         _ptr(out), _ptr(q), _ptr(cache), _ptr(sink), _ptr(seg_start), _ptr(seg_len),
         _ptr(seg_ctx), _ptr(block_tables), block_tables.shape[1], float(scale), S,

@@ -37,6 +37,7 @@ typedef float lr_f32x4 __attribute__((ext_vector_type(4)));
 #define LR_KVBLK 32
 #define LR_ROWS 64
 #define LR_PAD 8
+#define LR_PART_PAD 4  // a slice row is Dv values, running max, running sum, 2 unused
 
 template <int DKP, int DVP>
 __global__ __launch_bounds__(256) void latent_attention_rows_kernel(
@@ -48,7 +49,7 @@ __global__ __launch_bounds__(256) void latent_attention_rows_kernel(
     const int* __restrict__ seg_ctx,     // tokens of the sequence after this step
     const int* __restrict__ block_tables, int max_blocks, float scale, int H,
     int D, int Dv, int block_size, int nsplit,
-    float* __restrict__ partial) {  // [R * H, nsplit, Dv + 2] when nsplit > 1
+    float* __restrict__ partial) {  // [R * H, nsplit, Dv + 4] when nsplit > 1
   static_assert(DVP <= DKP, "values are a prefix of the key row");
   constexpr int DB = DVP / 16;
   constexpr int KB = DKP / 32;
@@ -229,7 +230,7 @@ __global__ __launch_bounds__(256) void latent_attention_rows_kernel(
 
   if (nsplit > 1) {
     // ---- partial result: unnormalised sums, running max and sum -------------------
-    const size_t stride = (size_t)Dv + 2;
+    const size_t stride = (size_t)Dv + LR_PART_PAD;
     if (row_valid && lg == 0) {
       float* pp = partial + (((size_t)lo * H + rho) * nsplit + z) * stride;
       pp[Dv] = m;
@@ -271,7 +272,10 @@ __global__ __launch_bounds__(256) void latent_attention_rows_kernel(
 
 
 // Merge the z-slices of every row: m* = max m_z, out = sum_z e^(m_z - m*) acc_z
-// / sum_z e^(m_z - m*) l_z.  One wave per row, lanes over the value entries.
+// / sum_z e^(m_z - m*) l_z.  One wave per row.  Lane z holds slice z's weight
+// (up to 64 slices); the lanes then own float4 columns of the value row and
+// add up the slices with independent 16-byte loads (slice rows are padded
+// to Dv + 4 floats so that they stay 16-byte aligned).
 __global__ __launch_bounds__(256) void latent_attention_rows_combine_kernel(
     uint16_t* __restrict__ out, const float* __restrict__ partial,
     const int* __restrict__ seg_start, const int* __restrict__ seg_len, int H,
@@ -279,26 +283,39 @@ __global__ __launch_bounds__(256) void latent_attention_rows_combine_kernel(
   const int s = blockIdx.y;
   const long nrows = (long)seg_len[s] * H;
   const long rho = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (rho >= nrows) return;
+  if (rho >= nrows) return;  // whole waves leave; no workgroup barrier below
   const int lane = threadIdx.x & 63;
   const size_t g = (size_t)seg_start[s] * H + rho;
-  const size_t stride = (size_t)Dv + 2;
+  const size_t stride = (size_t)Dv + LR_PART_PAD;
   const float* pp = partial + g * nsplit * stride;
-  float mstar = -INFINITY;
-  for (int zz = 0; zz < nsplit; ++zz) mstar = fmaxf(mstar, pp[zz * stride + Dv]);
-  float lsum = 0.f;
-  for (int zz = 0; zz < nsplit; ++zz) {
-    const float mz = pp[zz * stride + Dv];
-    if (mz != -INFINITY) lsum += __expf(mz - mstar) * pp[zz * stride + Dv + 1];
+  float mz = -INFINITY, lz = 0.f;
+  if (lane < nsplit) {
+    mz = pp[lane * stride + Dv];
+    lz = pp[lane * stride + Dv + 1];
   }
+  const float mstar = wave_reduce_max(mz);
+  const float wz = (mz == -INFINITY) ? 0.f : __expf(mz - mstar);
+  const float lsum = wave_reduce_sum(wz * lz);
   const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
-  for (int d = lane; d < Dv; d += 64) {
-    float a = 0.f;
+  for (int d0 = 0; d0 < Dv; d0 += 256) {  // uniform trip count: every lane feeds the shuffles
+    const int d = d0 + lane * 4;
+    const bool act = d < Dv;
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
     for (int zz = 0; zz < nsplit; ++zz) {
-      const float mz = pp[zz * stride + Dv];
-      if (mz != -INFINITY) a += __expf(mz - mstar) * pp[zz * stride + d];
+      const float w = __shfl(wz, zz, 64);
+      if (act) {
+        const f32x4 v = *reinterpret_cast<const f32x4*>(pp + zz * stride + d);
+        a0 += w * v[0];
+        a1 += w * v[1];
+        a2 += w * v[2];
+        a3 += w * v[3];
+      }
     }
-    out[g * Dv + d] = f32_to_bf16(a * inv);
+    if (!act) continue;
+    uint2 packed;
+    packed.x = (uint32_t)f32_to_bf16(a0 * inv) | ((uint32_t)f32_to_bf16(a1 * inv) << 16);
+    packed.y = (uint32_t)f32_to_bf16(a2 * inv) | ((uint32_t)f32_to_bf16(a3 * inv) << 16);
+    *reinterpret_cast<uint2*>(out + g * Dv + d) = packed;
   }
 }
 
