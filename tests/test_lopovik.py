@@ -68,6 +68,13 @@ CFG_L = {
     "layers": [lat(2, 8, 4, 8, 12, 12, dense(16)), lat(2, 8, 4, 8, 12, 12, moe(4, 3, 8))],
     "loop": {"start": 0, "stop": 2, "times": 1},
 }
+# no routed layer anywhere: on the GPU the engine pads such batches to whole
+# GEMM row multiples, so rows of no sequence travel through every kernel
+CFG_D = {
+    "architecture": "Lopovik", "vocab": 33, "width": 32, "norm": {"eps": 1e-5},
+    "layers": [lat(2, 8, 8, 8, 16, 24, dense(24)), lat(3, 4, 4, 6, 8, 12, None), lat(2, 8, 8, 8, 16, 24, dense(40))],
+    "loop": {"start": 1, "stop": 3, "times": 2},
+}
 # cache rows of three of the MFMA kernel's size classes (80, 128, 136 entries)
 CFG_C = {
     "architecture": "Lopovik", "vocab": 40, "width": 64, "norm": {"eps": 1e-5},
@@ -244,18 +251,27 @@ def test_whole_prompt_and_every_layer_run(model_a, oracle_a, device, dtype):
 
 
 @pytest.mark.parametrize("device", DEVICES)
-@pytest.mark.parametrize("which", ["b", "l"])
+@pytest.mark.parametrize("which", ["b", "l", "d"])
 def test_degenerate_sizes_and_loops(model_b, tmp_path, device, which):
     if which == "b":
         cfg, (path, W) = CFG_B, model_b
     else:
-        cfg = CFG_L
+        cfg = CFG_L if which == "l" else CFG_D
         W = make_checkpoint(cfg, 14)
-        path = write_model(tmp_path / "l", cfg, W)
+        path = write_model(tmp_path / which, cfg, W)
     toks = tokens_for(cfg, 40, 6)
     want = O.forward(cfg, W, toks)
     eng = make_engine(path, device, block_size=8)
+    assert get_model_config(path).is_moe == (which != "d")
     assert rel_err(replay_all(eng, "d", toks, [17, 1, 1, 2, 19]), want) < 2e-4
+    if which == "d":  # bf16 with padded batches, two requests side by side
+        eng = make_engine(path, device, torch.bfloat16 if device != "cpu" else torch.float32)
+        t2 = tokens_for(cfg, 21, 7)
+        r1 = eng.replay_step([("x", toks[:30], list(range(30))), ("y", t2[:20], list(range(20)))])
+        r2 = eng.replay_step([("x", toks[30:], list(range(10))), ("y", t2[20:], [0])], end=["x", "y"])
+        got_x = torch.cat([r1["x"], r2["x"]]).float().cpu()
+        got_y = torch.cat([r1["y"], r2["y"]]).float().cpu()
+        assert rel_err(got_x, want) < 6e-2 and rel_err(got_y, O.forward(cfg, W, t2)) < 6e-2
 
 
 @pytest.mark.parametrize("device", DEVICES)
