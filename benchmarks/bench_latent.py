@@ -122,6 +122,9 @@ def part_kernels(sizes) -> None:
             add("offset_norm_shift (two norms, token shift, state)", "",
                 timeit(lambda: ops.offset_norm_shift(x32, w, w, w, state, tok_seq, *segs, 1e-5)), T * H * 8)
             add("residual_add (both branches)", "", timeit(lambda: ops.residual_add(x32, y, y2)), T * H * 12)
+            # the add folded into the next layer's norms: + two addends in, the new residual out
+            add("offset_norm_shift with both branch outputs added on the way in", "",
+                timeit(lambda: ops.offset_norm_shift(x32, w, w, w, state, tok_seq, *segs, 1e-5, y, y2)), T * H * 16)
             add("fused_add_rms_norm (bf16 residual)", "offset_norm_shift + residual_add",
                 timeit(lambda: ops.fused_add_rms_norm(y, res16, torch.ones_like(w), 1e-5)), T * H * 8)
             up = torch.randn(T, FF, device=dev, dtype=bf)

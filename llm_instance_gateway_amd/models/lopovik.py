@@ -24,7 +24,9 @@ The residual stream is fp32 in every mode.
 Execution on the engine's flat batch, per layer run: one kernel for both
 norms and the shift, the mixer (fused input GEMM, latent prep kernel, query
 GEMMs, rotation, paged attention, value GEMM, gate, output GEMM), the
-feed-forward, one kernel adding both branch outputs into the residual.
+feed-forward.  Both branch outputs join the residual inside the NEXT layer's
+norm kernel (a kernel of its own only before a pass of the loop and before
+the final norm).
 """
 
 from __future__ import annotations
@@ -195,21 +197,32 @@ class LopovikForCausalLM(nn.Module):
     def forward(self, input_ids, positions, kv_caches, meta) -> torch.Tensor:
         eps = self.cfg.rms_norm_eps
         x0 = self.embed.index_select(0, input_ids).float()  # the embedding output, fp32
-        x = x0.clone() if self.loop_in is not None else x0
+        x = x0
+        # branch outputs of the layer before, not yet in the residual: the
+        # next layer's norm kernel adds them on its way in
+        pending = None
         for run, li in enumerate(self.run_order):
             layer = self.layers[li]
             if run in self.pass_starts:
+                if pending is not None:
+                    x = ops.residual_add(x.clone() if x is x0 else x, *pending)
+                    pending = None
                 x = F.linear(torch.cat([x, x0], dim=-1).to(self.dtype_), self.loop_in).float()
             lat_cache, shift_state = kv_caches[run]
-            h_mix, h_ff = ops.offset_norm_shift(
+            h_mix, h_ff, x = ops.offset_norm_shift(
                 x, layer.norm1, layer.norm2, layer.shift, shift_state, meta.tok_seq,
                 meta.seg_start, meta.seg_len, meta.seg_slot, meta.seg_fresh, eps,
+                *(pending or ()),
             )
             y = layer.mixer(h_mix, positions, (lat_cache,), meta)
             f = layer.mlp(h_ff, meta) if layer.mlp is not None else None
-            ops.residual_add(x, y, f)
+            pending = (y, f)
             if self.capture_residuals is not None:
+                x = ops.residual_add(x.clone() if x is x0 else x, y, f)
+                pending = None
                 self.capture_residuals.append(x.clone())
+        if pending is not None:
+            x = ops.residual_add(x.clone() if x is x0 else x, *pending)
         return ops.offset_rms_norm(x, self.final_norm, eps)
 
     def compute_logits(self, hidden: torch.Tensor, indices: torch.Tensor) -> torch.Tensor:

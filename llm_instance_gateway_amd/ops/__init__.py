@@ -712,31 +712,47 @@ def offset_rms_norm(x: torch.Tensor, w: torch.Tensor, eps: float) -> torch.Tenso
 
 
 def offset_norm_shift(
-    x, w_mix, w_ff, mu, state, tok_seq, seg_start, seg_len, seg_slot, seg_fresh, eps: float
+    x, w_mix, w_ff, mu, state, tok_seq, seg_start, seg_len, seg_slot, seg_fresh, eps: float,
+    add_a: Optional[torch.Tensor] = None, add_b: Optional[torch.Tensor] = None,
 ):
     """Both input norms of a parallel layer from one pass over the fp32
     residual x [R, H] (weights stored as offsets from one), with the mixer
     branch blended with the previous token's, h + (h_prev - h) * mu.  `state`
     [slots, H] fp32 carries each sequence's last unblended h between steps
-    and is updated in place.  w_ff None: no feed-forward branch.  Returns
-    (mixer input, feed-forward input or None) in w_mix's dtype; rows of no
-    segment are zero."""
+    and is updated in place.  w_ff None: no feed-forward branch.
+
+    add_a (and add_b): the previous layer's branch outputs, added on the way
+    in; the norms then read x + (add_a + add_b), which is returned as a new
+    residual tensor (x itself is left as it was).
+
+    Returns (mixer input, feed-forward input or None, residual) in w_mix's
+    dtype / fp32; rows of no segment are zero."""
     assert x.dtype == torch.float32 and state.dtype == torch.float32
+    assert add_b is None or add_a is not None
     if _use_hybrid(x):
         R, H = x.shape
         assert x.is_contiguous() and state.shape[1] == H and state.is_contiguous()
         hm = torch.empty(R, H, dtype=w_mix.dtype, device=x.device)
         hf = None if w_ff is None else torch.empty_like(hm)
+        x_out = x
+        if add_a is not None:
+            assert add_a.shape == x.shape and add_a.is_contiguous() and add_a.dtype == w_mix.dtype
+            assert add_b is None or (add_b.shape == x.shape and add_b.is_contiguous() and add_b.dtype == add_a.dtype)
+            x_out = torch.empty_like(x)
         _hl().lig_offset_norm_shift(
-            _ptr(hm), _ptr(hf), _ptr(x), _ptr(w_mix), _ptr(w_ff), _ptr(mu), _ptr(state),
-            _ptr(tok_seq), _ptr(seg_start), _ptr(seg_len), _ptr(seg_slot), _ptr(seg_fresh),
-            float(eps), R, H, _is_f32(w_mix), _stream(),
+            _ptr(hm), _ptr(hf), _ptr(x), _ptr(add_a), _ptr(add_b),
+            _ptr(x_out) if add_a is not None else None, _ptr(w_mix), _ptr(w_ff), _ptr(mu),
+            _ptr(state), _ptr(tok_seq), _ptr(seg_start), _ptr(seg_len), _ptr(seg_slot),
+            _ptr(seg_fresh), float(eps), R, H, _is_f32(w_mix), _stream(),
         )
-        return hm, hf
-    return torch_ref.offset_norm_shift(
+        return hm, hf, x_out
+    if add_a is not None:
+        x = torch_ref.residual_add(x.clone(), add_a, add_b)
+    hm, hf = torch_ref.offset_norm_shift(
         x, w_mix, w_ff, mu, state, tok_seq, seg_start, seg_len, seg_slot, seg_fresh, eps,
         w_mix.dtype,
     )
+    return hm, hf, x
 
 
 rotary_inv_freq = torch_ref.rotary_inv_freq

@@ -15,6 +15,11 @@
 // element are the same thread, so a segment of any length needs no second
 // launch.  All arithmetic is fp32; T is the storage type of the weights and
 // of the outputs.
+//
+// The previous layer's two branch outputs can be added on the way in
+// (x_new = x + (a + b), written to a second buffer so that neighbouring
+// workgroups still read the old rows): the residual add and the next layer's
+// norms are then one pass.
 
 #include "elem_types.h"
 
@@ -102,6 +107,8 @@ __global__ __launch_bounds__(SN_THREADS) void offset_norm_shift_kernel(
 template <typename T, int VPT>
 __global__ __launch_bounds__(SN_THREADS) void offset_norm_shift_vec_kernel(
     T* __restrict__ h_mix, T* __restrict__ h_ff, const float* __restrict__ x,
+    const T* __restrict__ add_a, const T* __restrict__ add_b,  // nullable addends
+    float* __restrict__ x_out,                                 // x + (a + b) when add_a
     const T* __restrict__ w_mix, const T* __restrict__ w_ff, const T* __restrict__ mu,
     float* __restrict__ state, const int* __restrict__ tok_seq,
     const int* __restrict__ seg_start, const int* __restrict__ seg_len,
@@ -118,6 +125,7 @@ __global__ __launch_bounds__(SN_THREADS) void offset_norm_shift_vec_kernel(
     for (int v = tid; v < nvec; v += SN_THREADS) {
       stn<4>(om + 4 * v, z);
       if (of) stn<4>(of + 4 * v, z);
+      if (add_a) stn<4>(x_out + (size_t)r * H + 4 * v, z);
     }
     return;
   }
@@ -128,8 +136,9 @@ __global__ __launch_bounds__(SN_THREADS) void offset_norm_shift_vec_kernel(
   const bool need_prev = shift && !first;
   const bool need_last = shift && first && r_last != r;
   const bool need_other = need_prev || need_last;  // never both
+  const size_t r_other = (size_t)(need_prev ? r - 1 : (need_last ? r_last : r));
   const float* xr = x + (size_t)r * H;
-  const float* xo = x + (size_t)(need_prev ? r - 1 : (need_last ? r_last : r)) * H;
+  const float* xo = x + r_other * H;
 
   float a[VPT][4], b[VPT][4];
   float sa = 0.f, sb = 0.f;
@@ -138,10 +147,25 @@ __global__ __launch_bounds__(SN_THREADS) void offset_norm_shift_vec_kernel(
     const int v = tid + k * SN_THREADS;
     if (v < nvec) {
       ldn<4>(xr + 4 * v, a[k]);
+      if (add_a) {
+        float p[4], q[4] = {0.f, 0.f, 0.f, 0.f};
+        ldn<4>(add_a + (size_t)r * H + 4 * v, p);
+        if (add_b) ldn<4>(add_b + (size_t)r * H + 4 * v, q);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) a[k][e] += p[e] + q[e];
+        stn<4>(x_out + (size_t)r * H + 4 * v, a[k]);
+      }
 #pragma unroll
       for (int e = 0; e < 4; ++e) sa += a[k][e] * a[k][e];
       if (need_other) {
         ldn<4>(xo + 4 * v, b[k]);
+        if (add_a) {  // the same sum the other row's workgroup stores
+          float p[4], q[4] = {0.f, 0.f, 0.f, 0.f};
+          ldn<4>(add_a + r_other * H + 4 * v, p);
+          if (add_b) ldn<4>(add_b + r_other * H + 4 * v, q);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) b[k][e] += p[e] + q[e];
+        }
 #pragma unroll
         for (int e = 0; e < 4; ++e) sb += b[k][e] * b[k][e];
       }
@@ -227,9 +251,10 @@ __global__ __launch_bounds__(SN_THREADS) void offset_rms_norm_kernel(
     st(out + (size_t)r * H + d, xr[d] * inv * (1.0f + ld(w + d)));
 }
 
-// x += a (+ b): the fp32 residual takes both branch outputs in one pass
+// out = x + (a + b): the fp32 residual takes both branch outputs in one pass
+// (out may be x itself)
 template <typename T, int N>
-__global__ void residual_add_kernel(float* __restrict__ x, const T* __restrict__ a,
+__global__ void residual_add_kernel(float* out, const float* x, const T* __restrict__ a,
                                     const T* __restrict__ b, long n) {
   for (long i = (blockIdx.x * (long)blockDim.x + threadIdx.x) * N; i < n;
        i += gridDim.x * (long)blockDim.x * N) {
@@ -239,13 +264,35 @@ __global__ void residual_add_kernel(float* __restrict__ x, const T* __restrict__
     if (b) ldn<N>(b + i, bv);
 #pragma unroll
     for (int k = 0; k < N; ++k) xv[k] += b ? av[k] + bv[k] : av[k];
-    stn<N>(x + i, xv);
+    stn<N>(out + i, xv);
   }
+}
+
+static void launch_residual_add(float* out, const float* x, const void* a, const void* b,
+                                long n, int is_f32, hipStream_t s) {
+  if (n <= 0) return;
+  const bool v4 = n % 4 == 0 && aligned16(out) && aligned16(x) && aligned16(a) &&
+                  (!b || aligned16(b));
+  const long items = v4 ? n / 4 : n;
+  long g = (items + 255) / 256;
+  const int grid = (int)(g > 65535 ? 65535 : g);
+#define LIG_RA(T, N)                                                            \
+  hipLaunchKernelGGL((residual_add_kernel<T, N>), dim3(grid), dim3(256), 0, s,  \
+                     out, x, (const T*)a, (const T*)b, n)
+  if (is_f32) {
+    if (v4) LIG_RA(float, 4); else LIG_RA(float, 1);
+  } else {
+    if (v4) LIG_RA(bf16s, 4); else LIG_RA(bf16s, 1);
+  }
+#undef LIG_RA
 }
 
 extern "C" {
 
+// add_a (and add_b) non-null: x_out = x + (add_a + add_b) and the norms read
+// x_out; x_out must be a buffer of its own.  add_a null: x_out is unused.
 void lig_offset_norm_shift(void* h_mix, void* h_ff, const float* x,
+                           const void* add_a, const void* add_b, float* x_out,
                            const void* w_mix, const void* w_ff, const void* mu,
                            float* state, const int* tok_seq, const int* seg_start,
                            const int* seg_len, const int* seg_slot,
@@ -253,14 +300,16 @@ void lig_offset_norm_shift(void* h_mix, void* h_ff, const float* x,
                            int is_f32, hipStream_t s) {
   if (R <= 0) return;
   const bool al = aligned16(h_mix) && aligned16(x) && aligned16(w_mix) && aligned16(state) &&
-                  (!h_ff || (aligned16(h_ff) && aligned16(w_ff))) && (!mu || aligned16(mu));
+                  (!h_ff || (aligned16(h_ff) && aligned16(w_ff))) && (!mu || aligned16(mu)) &&
+                  (!add_a || (aligned16(add_a) && aligned16(x_out))) && (!add_b || aligned16(add_b));
   if (H % 4 == 0 && H <= 4 * SN_THREADS * 8 && al) {
     const int vpt = (H / 4 + SN_THREADS - 1) / SN_THREADS;
 #define LIG_SNV(T, V)                                                            \
   hipLaunchKernelGGL((offset_norm_shift_vec_kernel<T, V>), dim3(R),              \
                      dim3(SN_THREADS), 0, s, (T*)h_mix, (T*)h_ff, x,             \
-                     (const T*)w_mix, (const T*)w_ff, (const T*)mu, state,       \
-                     tok_seq, seg_start, seg_len, seg_slot, seg_fresh, eps, H)
+                     (const T*)add_a, (const T*)add_b, x_out, (const T*)w_mix,   \
+                     (const T*)w_ff, (const T*)mu, state, tok_seq, seg_start,    \
+                     seg_len, seg_slot, seg_fresh, eps, H)
 #define LIG_SNV_PICK(T)                                                          \
   do {                                                                           \
     if (vpt <= 1) LIG_SNV(T, 1);                                                 \
@@ -272,6 +321,11 @@ void lig_offset_norm_shift(void* h_mix, void* h_ff, const float* x,
 #undef LIG_SNV_PICK
 #undef LIG_SNV
     return;
+  }
+  // any width: the add as a pass of its own, then the scalar kernel
+  if (add_a) {
+    launch_residual_add(x_out, x, add_a, add_b, (long)R * H, is_f32, s);
+    x = x_out;
   }
   if (is_f32)
     hipLaunchKernelGGL(offset_norm_shift_kernel<float>, dim3(R), dim3(SN_THREADS), 0, s,
@@ -298,20 +352,7 @@ void lig_offset_rms_norm(void* out, const float* x, const void* w, float eps,
 
 void lig_residual_add(float* x, const void* a, const void* b, long n, int is_f32,
                       hipStream_t s) {
-  if (n <= 0) return;
-  const bool v4 = n % 4 == 0 && aligned16(x) && aligned16(a) && (!b || aligned16(b));
-  const long items = v4 ? n / 4 : n;
-  long g = (items + 255) / 256;
-  const int grid = (int)(g > 65535 ? 65535 : g);
-#define LIG_RA(T, N)                                                            \
-  hipLaunchKernelGGL((residual_add_kernel<T, N>), dim3(grid), dim3(256), 0, s,  \
-                     x, (const T*)a, (const T*)b, n)
-  if (is_f32) {
-    if (v4) LIG_RA(float, 4); else LIG_RA(float, 1);
-  } else {
-    if (v4) LIG_RA(bf16s, 4); else LIG_RA(bf16s, 1);
-  }
-#undef LIG_RA
+  launch_residual_add(x, x, a, b, n, is_f32, s);
 }
 
 }  // extern "C"

@@ -81,7 +81,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "lig_paged_attention_general": [
             p, p, l, p, p, p, i, p, p, p, l, p, f, f, f, i, i, i, i, i, i, i, i, i, p,
         ],
-        "lig_offset_norm_shift": [p, p, p, p, p, p, p, p, p, p, p, p, f, i, i, i, p],
+        "lig_offset_norm_shift": [p, p, p, p, p, p, p, p, p, p, p, p, p, p, p, f, i, i, i, p],
         "lig_offset_rms_norm": [p, p, p, f, i, i, i, p],
         "lig_residual_add": [p, p, p, l, i, p],
         "lig_latent_kv_prep": [p, p, l, p, p, p, i, p, p, p, f, i, i, i, i, i, p],

@@ -357,10 +357,8 @@ def _rms_scale(x: torch.Tensor, eps: float) -> torch.Tensor:
 
 
 def residual_add(x, a, b=None) -> torch.Tensor:
-    """x += a (+ b), x fp32 in place."""
-    x.add_(a.float())
-    if b is not None:
-        x.add_(b.float())
+    """x += (a + b), x fp32 in place."""
+    x.add_(a.float() if b is None else a.float() + b.float())
     return x
 
 

@@ -42,9 +42,12 @@ def i32(v, device):
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H", [20, 257, 1028, 2560, 5000])  # scalar and 4-wide paths, 1..8 vectors per thread
-def test_offset_norm_shift_over_portions(device, dtype, H):
+@pytest.mark.parametrize("adds", [0, 1, 2])
+def test_offset_norm_shift_over_portions(device, dtype, H, adds):
     """Two sequences fed in portions of 1, 2 and more tokens through reused
-    slots; the blended rows equal the whole-sequence computation."""
+    slots; the blended rows equal the whole-sequence computation.  With
+    `adds` the rows arrive as a residual plus one or two branch outputs that
+    the kernel adds on its way in."""
     skip_cpu_bf16(device, dtype)
     g = torch.Generator().manual_seed(H)
     eps = 1e-4
@@ -73,10 +76,22 @@ def test_offset_norm_shift_over_portions(device, dtype, H):
         tok_seq.append(-1)  # a padding row
         rows.append(torch.randn(1, H, generator=g))
         x = torch.cat(rows).to(device)
-        hm, hf = ops.offset_norm_shift(
+        extra = []
+        if adds:
+            extra = [torch.randn(x.shape, generator=g).to(dtype).to(device) for _ in range(adds)]
+            x_eff, before = x, None
+            x = x_eff - sum(t.float() for t in extra)
+            before = x.clone()
+        hm, hf, x_new = ops.offset_norm_shift(
             x, w1.to(device), w2.to(device), mu.to(device), state, i32(tok_seq, device),
-            i32(s0, device), i32(sl, device), i32(slot, device), i32(fresh, device), eps,
+            i32(s0, device), i32(sl, device), i32(slot, device), i32(fresh, device), eps, *extra,
         )
+        if adds:
+            assert torch.equal(x, before), "the incoming residual is left as it was"
+            n_live = len(tok_seq) - 1
+            close(x_new[:n_live], x_eff[:n_live].double().cpu(), torch.float32)
+        else:
+            assert x_new is x
         assert hm.dtype == dtype and hf.dtype == dtype
         at = 0
         for k, _, lo, hi in step:
@@ -94,7 +109,7 @@ def test_offset_norm_without_feed_forward_branch(device):
     x = torch.randn(5, H, generator=g).to(device)
     w1, mu = torch.randn(H, generator=g).to(device), torch.rand(H, generator=g).to(device)
     state = torch.zeros(1, H, device=device)
-    hm, hf = ops.offset_norm_shift(
+    hm, hf, _ = ops.offset_norm_shift(
         x, w1, None, mu, state, i32([0] * 5, device), i32([0], device), i32([5], device),
         i32([0], device), i32([1], device), 1e-5,
     )
