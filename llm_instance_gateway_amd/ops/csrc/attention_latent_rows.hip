@@ -18,7 +18,8 @@
 // Consecutive lanes stage consecutive KEYS of one chunk column, so the
 // transposed 2-byte stores of a wave fall into consecutive LDS words; LDS
 // rows are padded by 16 bytes so that the 16-byte fragment reads of 16
-// different rows spread over all banks.
+// different rows spread over all banks.  The loads of the next tile are
+// issued before the current tile's arithmetic (one tile in registers).
 // Scores, running max and sum are fp32; an optional per-head sink starts a
 // row's running max at sink_h and its sum at one.
 //
@@ -38,6 +39,26 @@ typedef float lr_f32x4 __attribute__((ext_vector_type(4)));
 #define LR_ROWS 64
 #define LR_PAD 8
 #define LR_PART_PAD 4  // a slice row is Dv values, running max, running sum, 2 unused
+
+// NCH 16-byte chunks of one cache row (columns sd0, sd0 + 64, ...) into
+// registers; zeros for a key past the visible range (blk < 0) and for
+// columns at or past D.
+template <int NCH>
+LIG_DEVICE void lr_load_chunks(u16x8* stage, const uint16_t* __restrict__ cache, int blk,
+                               int t, int block_size, int D, int sd0) {
+  const uint16_t* rowp =
+      cache + ((size_t)(blk < 0 ? 0 : blk) * block_size + (t % block_size)) * D;
+#pragma unroll
+  for (int j = 0; j < NCH; ++j) {
+    const int d0 = sd0 + j * 64;
+    if (blk >= 0 && d0 < D) {
+      stage[j] = *reinterpret_cast<const u16x8*>(rowp + d0);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) stage[j][e] = 0;
+    }
+  }
+}
 
 template <int DKP, int DVP>
 __global__ __launch_bounds__(256) void latent_attention_rows_kernel(
@@ -120,28 +141,46 @@ __global__ __launch_bounds__(256) void latent_attention_rows_kernel(
     kv_hi = min(kv_end, kv_lo + per * LR_KVBLK);
   }
 
+  // Staging is software-pipelined: a thread always stages the same key row of
+  // a tile (256 threads = 8 chunk columns x 32 keys, NCH column groups), so it
+  // needs ONE block-table entry per tile.  The chunks of tile i+1 are loaded
+  // into registers, and the table entry of tile i+2 is fetched, while tile i
+  // is being multiplied; they are written to LDS at the top of the next turn.
+  constexpr int NCH = DKP / 64;
+  const int srow = tid % LR_KVBLK;
+  const int sd0 = (tid / LR_KVBLK) * 8;
+  u16x8 stage[NCH];
+  int blk_next;
+  {
+    const int t = kv_lo + srow;
+    const int blk = (kv_lo < kv_hi && t < kv_end) ? bt[t / block_size] : -1;
+    lr_load_chunks<NCH>(stage, cache, blk, t, block_size, D, sd0);
+    const int t2 = t + LR_KVBLK;
+    blk_next = (kv_lo + LR_KVBLK < kv_hi && t2 < kv_end) ? bt[t2 / block_size] : -1;
+  }
+
   for (int kv0 = kv_lo; kv0 < kv_hi; kv0 += LR_KVBLK) {
-    // ---- staging: one load per 16-byte chunk, stored row-major and transposed ----
-    for (int c = tid; c < LR_KVBLK * (DKP / 8); c += 256) {
-      const int row = c % LR_KVBLK;
-      const int d0 = (c / LR_KVBLK) * 8;
-      const int t = kv0 + row;
-      u16x8 kval;
-      if (t < kv_end && d0 < D) {
-        const size_t base =
-            ((size_t)bt[t / block_size] * block_size + (t % block_size)) * D + d0;
-        kval = *reinterpret_cast<const u16x8*>(cache + base);
-      } else {
+    // ---- registers -> LDS: row-major for S^T = K Q^T, transposed for O += P V ----
 #pragma unroll
-        for (int e = 0; e < 8; ++e) kval[e] = 0;
-      }
-      *reinterpret_cast<u16x8*>(&sm.K[row][d0]) = kval;
+    for (int j = 0; j < NCH; ++j) {
+      const int d0 = sd0 + j * 64;
+      const u16x8 kval = stage[j];
+      *reinterpret_cast<u16x8*>(&sm.K[srow][d0]) = kval;
       if (d0 < DVP) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) sm.VT[d0 + e][row] = (d0 + e < Dv) ? kval[e] : (uint16_t)0;
+        for (int e = 0; e < 8; ++e) sm.VT[d0 + e][srow] = (d0 + e < Dv) ? kval[e] : (uint16_t)0;
       }
     }
     __syncthreads();
+    {  // prefetch the next tile (loads stay in flight through the arithmetic below)
+      const int kvn = kv0 + LR_KVBLK;
+      if (kvn < kv_hi) {
+        const int t = kvn + srow;
+        lr_load_chunks<NCH>(stage, cache, blk_next, t, block_size, D, sd0);
+        const int t2 = t + LR_KVBLK;
+        blk_next = (kvn + LR_KVBLK < kv_hi && t2 < kv_end) ? bt[t2 / block_size] : -1;
+      }
+    }
 
     if (wave_active) {
     // ---- S^T = K Q^T ----------------------------------------------------------
