@@ -340,15 +340,28 @@ __global__ __launch_bounds__(256) void latent_attention_rows_combine_kernel(
     const int d = d0 + lane * 4;
     const bool act = d < Dv;
     float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
-    for (int zz = 0; zz < nsplit; ++zz) {
-      const float w = __shfl(wz, zz, 64);
-      if (act) {
-        const f32x4 v = *reinterpret_cast<const f32x4*>(pp + zz * stride + d);
-        a0 += w * v[0];
-        a1 += w * v[1];
-        a2 += w * v[2];
-        a3 += w * v[3];
+    const float* col = pp + (act ? d : 0);
+    int zz = 0;
+    for (; zz + 4 <= nsplit; zz += 4) {  // four slices' loads in flight at a time
+      f32x4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) v[u] = *reinterpret_cast<const f32x4*>(col + (zz + u) * stride);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const float w = __shfl(wz, zz + u, 64);
+        a0 += w * v[u][0];
+        a1 += w * v[u][1];
+        a2 += w * v[u][2];
+        a3 += w * v[u][3];
       }
+    }
+    for (; zz < nsplit; ++zz) {
+      const float w = __shfl(wz, zz, 64);
+      const f32x4 v = *reinterpret_cast<const f32x4*>(col + zz * stride);
+      a0 += w * v[0];
+      a1 += w * v[1];
+      a2 += w * v[2];
+      a3 += w * v[3];
     }
     if (!act) continue;
     uint2 packed;
